@@ -1,0 +1,123 @@
+"""Engine configuration: frozen, validated sub-configs composed in ``KVCoreConfig``.
+
+Names and meanings follow the reference's kvcore/config.py:15-192 where it has them;
+sparse-KV and prefix-cache settings have no counterpart here.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from pathlib import Path
+
+DTYPE_NAMES = {
+    "bfloat16": "bfloat16",
+    "bf16": "bfloat16",
+    "float32": "float32",
+    "fp32": "float32",
+    "float": "float32",
+}
+
+
+def canonical_dtype(name: str | None) -> str | None:
+    """``"bfloat16"`` or ``"float32"`` from any of their usual spellings."""
+    if name is None:
+        return None
+    key = str(name).replace("torch.", "").lower()
+    if key not in DTYPE_NAMES:
+        raise ValueError(f"unsupported dtype {name!r}; supported: bfloat16, float32")
+    return DTYPE_NAMES[key]
+
+
+@dataclass(frozen=True)
+class ModelConfig:
+    """Reference: config.py:15-30.  ``dtype`` None means: config.json's ``dtype`` if it
+    is one of ours, else bfloat16."""
+
+    model: str | Path
+    tokenizer: str | Path | None = None
+    dtype: str | None = None
+    max_model_len: int | None = None
+
+    def __post_init__(self) -> None:
+        if self.max_model_len is not None and self.max_model_len <= 0:
+            raise ValueError(f"max_model_len must be positive, got {self.max_model_len}")
+        object.__setattr__(self, "dtype", canonical_dtype(self.dtype))
+
+
+@dataclass(frozen=True)
+class LoadConfig:
+    """Reference: config.py:33-40.  ``load_format`` is ``"safetensors"`` (read the
+    folder's files) or ``"random"`` (fill every parameter from ``seed``; the folder
+    then needs only config.json).  ``strict`` also refuses unexpected tensors, which
+    the reference drops silently (kvcore/model/model_utils.py:65-76)."""
+
+    load_format: str = "safetensors"
+    strict: bool = True
+    seed: int = 0
+
+    def __post_init__(self) -> None:
+        if self.load_format not in ("safetensors", "random", "auto"):
+            raise ValueError(f"load_format must be 'safetensors' or 'random', got {self.load_format!r}")
+
+
+@dataclass(frozen=True)
+class CacheConfig:
+    """Reference: config.py:43-60.  ``num_gpu_blocks`` counts pages including the
+    reserved null page; when given it wins over profiling."""
+
+    block_size: int = 16
+    num_gpu_blocks: int | None = None
+    profile_kv_cache: bool = True
+    gpu_memory_utilization: float = 0.9
+
+    def __post_init__(self) -> None:
+        if self.block_size <= 0:
+            raise ValueError(f"block_size must be positive, got {self.block_size}")
+        if self.num_gpu_blocks is not None and self.num_gpu_blocks <= 1:
+            raise ValueError(f"num_gpu_blocks must exceed 1 (page 0 is reserved), got {self.num_gpu_blocks}")
+        if not 0 < self.gpu_memory_utilization <= 1:
+            raise ValueError(
+                f"gpu_memory_utilization must be in (0, 1], got {self.gpu_memory_utilization}"
+            )
+
+
+@dataclass(frozen=True)
+class SchedulerConfig:
+    """Reference: config.py:63-93 (same five names, same validation)."""
+
+    max_num_seqs: int = 8
+    max_num_scheduled_tokens: int = 512
+    max_num_partial_prefills: int = 1
+    max_long_partial_prefills: int = 1
+    long_prefill_token_threshold: int = 0
+
+    def __post_init__(self) -> None:
+        for name in (
+            "max_num_seqs", "max_num_scheduled_tokens",
+            "max_num_partial_prefills", "max_long_partial_prefills",
+        ):
+            if getattr(self, name) <= 0:
+                raise ValueError(f"{name} must be positive, got {getattr(self, name)}")
+        if self.long_prefill_token_threshold < 0:
+            raise ValueError(
+                f"long_prefill_token_threshold must be non-negative, got {self.long_prefill_token_threshold}"
+            )
+
+
+@dataclass(frozen=True)
+class DeviceConfig:
+    """Reference: config.py:160-162.  ROCm torch names HIP devices ``cuda``."""
+
+    device: str = "cuda:0"
+    use_hip_graphs: bool = True
+
+
+@dataclass(frozen=True)
+class KVCoreConfig:
+    """Reference: config.py:165-192."""
+
+    model_config: ModelConfig
+    load_config: LoadConfig = field(default_factory=LoadConfig)
+    cache_config: CacheConfig = field(default_factory=CacheConfig)
+    scheduler_config: SchedulerConfig = field(default_factory=SchedulerConfig)
+    device_config: DeviceConfig = field(default_factory=DeviceConfig)

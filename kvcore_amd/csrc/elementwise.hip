@@ -1,0 +1,361 @@
+// Row-wise and element-wise kernels: embedding, RMSNorm with the residual sum,
+// SiLU-mul, row gather, rotary tables, rotation fused with the paged K/V write,
+// block-table updates.  All arithmetic is float32; storage is float32 or bfloat16.
+
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+#include <string>
+
+#include "device_utils.h"
+#include "kvcore_hip.h"
+
+using namespace kvc;
+
+// ------------------------------------------------------------------ error plumbing
+static thread_local std::string g_last_error;
+
+int kvc_fail(const char* message) {
+  g_last_error = message;
+  return -1;
+}
+
+int kvc_check_launch(const char* what) {
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    g_last_error = std::string(what) + ": " + hipGetErrorString(err);
+    return -2;
+  }
+  return 0;
+}
+
+extern "C" const char* kvc_last_error(void) { return g_last_error.c_str(); }
+extern "C" int kvc_version(void) { return 1; }
+
+static inline hipStream_t S(kvc_stream s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ------------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ residual, const T* __restrict__ table,
+                             const int32_t* __restrict__ ids, int H, int V) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  float* out = residual + static_cast<int64_t>(t) * H;
+  if (id < 0 || id >= V) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = __uint_as_float(0x7fc00000u);
+    return;
+  }
+  const T* row = table + static_cast<int64_t>(id) * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_float(row[i]);
+}
+
+extern "C" int kvc_embed(float* residual, const void* table, const int32_t* ids, int T, int H,
+                         int V, int dtype, kvc_stream stream) {
+  if (T < 0 || H <= 0 || V <= 0) return kvc_fail("kvc_embed: bad sizes");
+  if (T == 0) return 0;
+  KVC_DISPATCH_DTYPE(dtype, Tp, hipLaunchKernelGGL(embed_kernel<Tp>, dim3(T), dim3(256), 0,
+                                                   S(stream), residual,
+                                                   static_cast<const Tp*>(table), ids, H, V));
+  return kvc_check_launch("kvc_embed");
+}
+
+// -------------------------------------------------------------------------- RMSNorm
+// One block per row.  Pass 1 forms the residual sum in float32, stores it and
+// accumulates the squares; pass 2 reads the sums back (each thread its own) and scales.
+template <typename T>
+__global__ void add_rmsnorm_kernel(T* __restrict__ out, float* __restrict__ residual,
+                                   const T* __restrict__ delta, const float* __restrict__ weight,
+                                   float eps, int H) {
+  __shared__ float scratch[16];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * H;
+  float* r = residual + base;
+  float ss = 0.f;
+  if (delta != nullptr) {
+    const T* dl = delta + base;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      const float v = r[i] + to_float(dl[i]);
+      r[i] = v;
+      ss += v * v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      const float v = r[i];
+      ss += v * v;
+    }
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = rsqrtf(total / static_cast<float>(H) + eps);
+  T* o = out + base;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = from_float<T>(weight[i] * (r[i] * inv));
+}
+
+extern "C" int kvc_add_rmsnorm(void* out, float* residual, const void* delta, const float* weight,
+                               float eps, int T, int H, int dtype, kvc_stream stream) {
+  if (T < 0 || H <= 0) return kvc_fail("kvc_add_rmsnorm: bad sizes");
+  if (T == 0) return 0;
+  KVC_DISPATCH_DTYPE(dtype, Tp,
+                     hipLaunchKernelGGL(add_rmsnorm_kernel<Tp>, dim3(T), dim3(256), 0, S(stream),
+                                        static_cast<Tp*>(out), residual,
+                                        static_cast<const Tp*>(delta), weight, eps, H));
+  return kvc_check_launch("kvc_add_rmsnorm");
+}
+
+template <typename T>
+__global__ void rmsnorm_kernel(T* __restrict__ out, const T* __restrict__ x,
+                               const float* __restrict__ weight, float eps, int H,
+                               int64_t x_stride, int64_t out_stride) {
+  __shared__ float scratch[16];
+  const T* xr = x + static_cast<int64_t>(blockIdx.x) * x_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float v = to_float(xr[i]);
+    ss += v * v;
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = rsqrtf(total / static_cast<float>(H) + eps);
+  T* o = out + static_cast<int64_t>(blockIdx.x) * out_stride;
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    o[i] = from_float<T>(weight[i] * (to_float(xr[i]) * inv));
+}
+
+extern "C" int kvc_rmsnorm(void* out, const void* x, const float* weight, float eps, int T, int H,
+                           int64_t x_stride, int64_t out_stride, int dtype, kvc_stream stream) {
+  if (T < 0 || H <= 0 || x_stride < H || out_stride < H) return kvc_fail("kvc_rmsnorm: bad sizes");
+  if (T == 0) return 0;
+  KVC_DISPATCH_DTYPE(dtype, Tp,
+                     hipLaunchKernelGGL(rmsnorm_kernel<Tp>, dim3(T), dim3(256), 0, S(stream),
+                                        static_cast<Tp*>(out), static_cast<const Tp*>(x), weight,
+                                        eps, H, x_stride, out_stride));
+  return kvc_check_launch("kvc_rmsnorm");
+}
+
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                    int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) residual[i] += to_float(delta[i]);
+}
+
+extern "C" int kvc_residual_add(float* residual, const void* delta, int T, int H, int dtype,
+                                kvc_stream stream) {
+  if (T < 0 || H <= 0) return kvc_fail("kvc_residual_add: bad sizes");
+  const int64_t n = static_cast<int64_t>(T) * H;
+  if (n == 0) return 0;
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  KVC_DISPATCH_DTYPE(dtype, Tp,
+                     hipLaunchKernelGGL(residual_add_kernel<Tp>, dim3(blocks), dim3(256), 0,
+                                        S(stream), residual, static_cast<const Tp*>(delta), n));
+  return kvc_check_launch("kvc_residual_add");
+}
+
+// ------------------------------------------------------------------------- SiLU-mul
+template <typename T>
+__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gate_up, int I,
+                                int64_t n) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t t = idx / I;
+  const int i = static_cast<int>(idx - t * I);
+  const T* row = gate_up + t * 2 * I;
+  const float g = to_float(row[i]);
+  const float u = to_float(row[I + i]);
+  const float s = g / (1.f + expf(-g));
+  out[idx] = from_float<T>(s * u);
+}
+
+extern "C" int kvc_silu_mul(void* out, const void* gate_up, int T, int I, int dtype,
+                            kvc_stream stream) {
+  if (T < 0 || I <= 0) return kvc_fail("kvc_silu_mul: bad sizes");
+  const int64_t n = static_cast<int64_t>(T) * I;
+  if (n == 0) return 0;
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  KVC_DISPATCH_DTYPE(dtype, Tp,
+                     hipLaunchKernelGGL(silu_mul_kernel<Tp>, dim3(blocks), dim3(256), 0, S(stream),
+                                        static_cast<Tp*>(out), static_cast<const Tp*>(gate_up), I,
+                                        n));
+  return kvc_check_launch("kvc_silu_mul");
+}
+
+// ----------------------------------------------------------------------- row gather
+template <typename TI, typename TO>
+__global__ void gather_rows_kernel(TO* __restrict__ out, const TI* __restrict__ in,
+                                   const int32_t* __restrict__ rows, int H) {
+  const int s = blockIdx.x;
+  const TI* src = in + static_cast<int64_t>(rows[s]) * H;
+  TO* dst = out + static_cast<int64_t>(s) * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = from_float<TO>(to_float(src[i]));
+}
+
+extern "C" int kvc_gather_rows(void* out, const void* in, const int32_t* rows, int S_, int H,
+                               int in_dtype, int out_dtype, kvc_stream stream) {
+  if (S_ < 0 || H <= 0) return kvc_fail("kvc_gather_rows: bad sizes");
+  if (S_ == 0) return 0;
+  if (in_dtype == 0 && out_dtype == 0) {
+    hipLaunchKernelGGL((gather_rows_kernel<float, float>), dim3(S_), dim3(256), 0, S(stream),
+                       static_cast<float*>(out), static_cast<const float*>(in), rows, H);
+  } else if (in_dtype == 1 && out_dtype == 1) {
+    hipLaunchKernelGGL((gather_rows_kernel<bf16_t, bf16_t>), dim3(S_), dim3(256), 0, S(stream),
+                       static_cast<bf16_t*>(out), static_cast<const bf16_t*>(in), rows, H);
+  } else if (in_dtype == 0 && out_dtype == 1) {
+    hipLaunchKernelGGL((gather_rows_kernel<float, bf16_t>), dim3(S_), dim3(256), 0, S(stream),
+                       static_cast<bf16_t*>(out), static_cast<const float*>(in), rows, H);
+  } else if (in_dtype == 1 && out_dtype == 0) {
+    hipLaunchKernelGGL((gather_rows_kernel<bf16_t, float>), dim3(S_), dim3(256), 0, S(stream),
+                       static_cast<float*>(out), static_cast<const bf16_t*>(in), rows, H);
+  } else {
+    return kvc_fail("kvc_gather_rows: unknown dtype code");
+  }
+  return kvc_check_launch("kvc_gather_rows");
+}
+
+template <typename T>
+__global__ void to_float_kernel(float* __restrict__ out, const T* __restrict__ in, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = to_float(in[i]);
+}
+
+extern "C" int kvc_to_float(float* out, const void* in, int64_t n, int dtype, kvc_stream stream) {
+  if (n < 0) return kvc_fail("kvc_to_float: bad size");
+  if (n == 0) return 0;
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  KVC_DISPATCH_DTYPE(dtype, Tp,
+                     hipLaunchKernelGGL(to_float_kernel<Tp>, dim3(blocks), dim3(256), 0, S(stream),
+                                        out, static_cast<const Tp*>(in), n));
+  return kvc_check_launch("kvc_to_float");
+}
+
+// -------------------------------------------------------------------- rotary tables
+__global__ void rope_table_kernel(float* __restrict__ cos_out, float* __restrict__ sin_out,
+                                  const int32_t* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, int half, int64_t n) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t t = idx / half;
+  const int j = static_cast<int>(idx - t * half);
+  const float angle = static_cast<float>(positions[t]) * inv_freq[j];
+  float s, c;
+  sincosf(angle, &s, &c);
+  cos_out[idx] = c;
+  sin_out[idx] = s;
+}
+
+extern "C" int kvc_rope_table(float* cos_out, float* sin_out, const int32_t* positions,
+                              const float* inv_freq, int T, int half, kvc_stream stream) {
+  if (T < 0 || half <= 0) return kvc_fail("kvc_rope_table: bad sizes");
+  const int64_t n = static_cast<int64_t>(T) * half;
+  if (n == 0) return 0;
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  hipLaunchKernelGGL(rope_table_kernel, dim3(blocks), dim3(256), 0, S(stream), cos_out, sin_out,
+                     positions, inv_freq, half, n);
+  return kvc_check_launch("kvc_rope_table");
+}
+
+// ------------------------------------------------- rotation fused with the K/V write
+// One block per token.  Work items: (head, pair) rotations for the nh + nkv rotated
+// heads, then pass-through elements (beyond rot_dim, and all of v).
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cache,
+                                     T* __restrict__ v_cache, const float* __restrict__ cos_tab,
+                                     const float* __restrict__ sin_tab, int rot_dim,
+                                     int interleaved, const int32_t* __restrict__ positions,
+                                     const int32_t* __restrict__ token_req,
+                                     const int32_t* __restrict__ slots,
+                                     const int32_t* __restrict__ table, int table_stride, int nh,
+                                     int nkv, int d, int page_size, int num_pages, int write_kv) {
+  const int t = blockIdx.x;
+  const int req = token_req[t];
+  if (req < 0) return;
+  const int pos = positions[t];
+  const int half = rot_dim / 2;
+  T* row = qkv + static_cast<int64_t>(t) * (nh + 2 * nkv) * d;
+
+  int64_t cache_base = -1;  // element offset of [page, kv head 0, pos % page_size, 0]
+  if (write_kv) {
+    const int slot = slots[req];
+    const int page = table[static_cast<int64_t>(slot) * table_stride + pos / page_size];
+    if (page > 0 && page < num_pages)
+      cache_base = (static_cast<int64_t>(page) * nkv * page_size + pos % page_size) * d;
+  }
+  const int64_t head_step = static_cast<int64_t>(page_size) * d;  // between kv heads in a page
+
+  const float* cs = cos_tab + static_cast<int64_t>(t) * half;
+  const float* sn = sin_tab + static_cast<int64_t>(t) * half;
+
+  // rotations: heads 0..nh-1 are q, nh..nh+nkv-1 are k
+  const int n_rot = (nh + nkv) * half;
+  for (int w = threadIdx.x; w < n_rot; w += blockDim.x) {
+    const int head = w / half;
+    const int j = w - head * half;
+    const int i0 = interleaved ? 2 * j : j;
+    const int i1 = interleaved ? 2 * j + 1 : j + half;
+    T* hp = row + static_cast<int64_t>(head) * d;
+    const float x0 = to_float(hp[i0]);
+    const float x1 = to_float(hp[i1]);
+    const float c = cs[j], s = sn[j];
+    const T y0 = from_float<T>(x0 * c - x1 * s);
+    const T y1 = from_float<T>(x1 * c + x0 * s);
+    hp[i0] = y0;
+    hp[i1] = y1;
+    if (head >= nh && cache_base >= 0) {
+      T* kc = k_cache + cache_base + (head - nh) * head_step;
+      kc[i0] = y0;
+      kc[i1] = y1;
+    }
+  }
+  if (cache_base < 0) return;
+  // k elements beyond the rotated part
+  const int tail = d - rot_dim;
+  if (tail > 0) {
+    for (int w = threadIdx.x; w < nkv * tail; w += blockDim.x) {
+      const int head = w / tail;
+      const int i = rot_dim + (w - head * tail);
+      k_cache[cache_base + head * head_step + i] = row[static_cast<int64_t>(nh + head) * d + i];
+    }
+  }
+  // v
+  for (int w = threadIdx.x; w < nkv * d; w += blockDim.x) {
+    const int head = w / d;
+    const int i = w - head * d;
+    v_cache[cache_base + head * head_step + i] = row[static_cast<int64_t>(nh + nkv + head) * d + i];
+  }
+}
+
+extern "C" int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_tab,
+                                 const float* sin_tab, int rot_dim, int interleaved,
+                                 const int32_t* positions, const int32_t* token_req,
+                                 const int32_t* slots, const int32_t* table, int table_stride,
+                                 int T, int nh, int nkv, int d, int page_size, int num_pages,
+                                 int write_kv, int dtype, kvc_stream stream) {
+  if (T < 0 || nh <= 0 || nkv <= 0 || d <= 0 || page_size <= 0 || num_pages <= 0)
+    return kvc_fail("kvc_rope_kv_write: bad sizes");
+  if (rot_dim < 0 || rot_dim > d || (rot_dim & 1))
+    return kvc_fail("kvc_rope_kv_write: rot_dim must be even and at most the head size");
+  if (T == 0) return 0;
+  KVC_DISPATCH_DTYPE(
+      dtype, Tp,
+      hipLaunchKernelGGL(rope_kv_write_kernel<Tp>, dim3(T), dim3(256), 0, S(stream),
+                         static_cast<Tp*>(qkv), static_cast<Tp*>(k_cache),
+                         static_cast<Tp*>(v_cache), cos_tab, sin_tab, rot_dim, interleaved,
+                         positions, token_req, slots, table, table_stride, nh, nkv, d, page_size,
+                         num_pages, write_kv));
+  return kvc_check_launch("kvc_rope_kv_write");
+}
+
+// ------------------------------------------------------------- block-table updates
+__global__ void table_update_kernel(int32_t* __restrict__ table, int table_stride, int table_rows,
+                                    const int32_t* __restrict__ triples, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int row = triples[3 * i], col = triples[3 * i + 1], val = triples[3 * i + 2];
+  if (row < 0 || row >= table_rows || col < 0 || col >= table_stride) return;
+  table[static_cast<int64_t>(row) * table_stride + col] = val;
+}
+
+extern "C" int kvc_table_update(int32_t* table, int table_stride, int table_rows,
+                                const int32_t* triples, int n, kvc_stream stream) {
+  if (n < 0 || table_stride <= 0 || table_rows <= 0) return kvc_fail("kvc_table_update: bad sizes");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(table_update_kernel, dim3((n + 255) / 256), dim3(256), 0, S(stream), table,
+                     table_stride, table_rows, triples, n);
+  return kvc_check_launch("kvc_table_update");
+}

@@ -1,0 +1,96 @@
+// C interface of the gfx950 kernel library.  Every function launches on the given
+// stream and returns at once; 0 means the launch was accepted, a negative value
+// means the arguments were refused (kvc_last_error() holds the reason) and nothing
+// was launched.  Pointers are device pointers unless named host_*.
+//
+// dtype codes: 0 = float32, 1 = bfloat16.  "dt" in a comment means that type.
+#pragma once
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* kvc_stream;
+
+const char* kvc_last_error(void);
+int kvc_version(void);
+
+// residual[t, :] = float(table[ids[t], :]); an id outside [0, V) gives a NaN row.
+int kvc_embed(float* residual, const void* table, const int32_t* ids, int T, int H, int V,
+              int dtype, kvc_stream stream);
+
+// residual += delta (skipped when delta is null); out = weight * residual *
+// rsqrt(mean(residual^2) + eps), rounded to dt.  residual stays float32.
+int kvc_add_rmsnorm(void* out, float* residual, const void* delta, const float* weight,
+                    float eps, int T, int H, int dtype, kvc_stream stream);
+
+// out = weight * x * rsqrt(mean(x^2) + eps) on rows of dt (no residual), row strides given.
+int kvc_rmsnorm(void* out, const void* x, const float* weight, float eps, int T, int H,
+                int64_t x_stride, int64_t out_stride, int dtype, kvc_stream stream);
+
+// residual += delta, nothing else.
+int kvc_residual_add(float* residual, const void* delta, int T, int H, int dtype,
+                     kvc_stream stream);
+
+// out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i].
+int kvc_silu_mul(void* out, const void* gate_up, int T, int I, int dtype, kvc_stream stream);
+
+// out[s, :] = in[rows[s], :]; `in` may be float32 (in_dtype 0) while out is dt.
+int kvc_gather_rows(void* out, const void* in, const int32_t* rows, int S, int H, int in_dtype,
+                    int out_dtype, kvc_stream stream);
+
+// out = float(in) elementwise (n values).
+int kvc_to_float(float* out, const void* in, int64_t n, int dtype, kvc_stream stream);
+
+// cos/sin[t, j] of the angle float(positions[t]) * inv_freq[j], j < half.
+int kvc_rope_table(float* cos_out, float* sin_out, const int32_t* positions,
+                   const float* inv_freq, int T, int half, kvc_stream stream);
+
+// Rotates the first rot_dim elements of every q and k head of qkv [T, (nh+2nkv)*d] in
+// place (pairs (j, j+rot_dim/2), or (2j, 2j+1) when interleaved), then, when write_kv is
+// set, stores the rotated k and the v of token t at its page slot:
+//   slot row  = slots[token_req[t]], page = table[row, pos / page_size],
+//   cache[page, kv_head, pos % page_size, :].
+// Tokens with token_req < 0 are left alone.
+int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_tab,
+                      const float* sin_tab, int rot_dim, int interleaved,
+                      const int32_t* positions, const int32_t* token_req, const int32_t* slots,
+                      const int32_t* table, int table_stride, int T, int nh, int nkv, int d,
+                      int page_size, int num_pages, int write_kv, int dtype, kvc_stream stream);
+
+// Attention of every token over its request's cache: token t at position p sees keys
+// max(0, p - window + 1) .. p (window <= 0: all), read through the block table.
+// q is [T, nh, d] with q_stride elements between tokens; out is [T, nh*d].
+int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* k_cache,
+                        const void* v_cache, const int32_t* table, int table_stride,
+                        const int32_t* positions, const int32_t* token_req,
+                        const int32_t* slots, int T, int nh, int nkv, int d, int page_size,
+                        int num_pages, float scale, int window, int dtype, kvc_stream stream);
+
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) in float32 with float32 products and sums;
+// each element is one running sum over k = 0..K-1, whatever M is.
+int kvc_gemm_f32(float* C, const float* A, const float* W, const float* bias, int M, int N,
+                 int K, int64_t lda, int64_t ldc, kvc_stream stream);
+
+// table[triples[3i], triples[3i+1]] = triples[3i+2] for i < n.
+int kvc_table_update(int32_t* table, int table_stride, int table_rows, const int32_t* triples,
+                     int n, kvc_stream stream);
+
+// out[s] = index of the largest logit of row s (the lowest index among equals).
+int kvc_argmax(int32_t* out, const float* logits, int S, int V, int64_t row_stride,
+               kvc_stream stream);
+
+// Per row s: temperature[s] < 1e-5 gives the argmax; otherwise
+// argmax_v(logits[v] / temperature - log(e_v)), e_v exponential noise keyed by
+// (seed_lo[s], seed_hi[s], index[s], v), over the entries that top_k[s] (<= 0: all) and
+// top_p[s] (>= 1: all) keep.
+int kvc_sample(int32_t* out, const float* logits, int S, int V, int64_t row_stride,
+               const float* temperature, const int32_t* top_k, const float* top_p,
+               const uint32_t* seed_lo, const uint32_t* seed_hi, const uint32_t* index,
+               kvc_stream stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,199 @@
+// Sampling over float32 logits: one block of 1024 threads per row.
+//
+// Greedy is the argmax (lowest index among equals).  Otherwise the row is divided by
+// its temperature; top-k and top-p become a value threshold found by 32 halvings over
+// the order-preserving integer image of float32 (no sort); the token is
+// argmax_v(z_v - log(e_v)) with e_v = -log(u_v) exponential noise, which is the same
+// draw as argmax_v(softmax(z)_v / e_v).  u_v comes from 32-bit integer mixing of
+// (seed, output index, v), so a row's draw depends on nothing else in the batch.
+
+#include <hip/hip_runtime.h>
+
+#include "device_utils.h"
+#include "kvcore_hip.h"
+
+using namespace kvc;
+
+namespace {
+
+constexpr int kThreads = 1024;
+constexpr float kGreedyEps = 1e-5f;
+
+__device__ __forceinline__ uint32_t fmix(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x85EBCA6Bu;
+  x ^= x >> 13;
+  x *= 0xC2B2AE35u;
+  x ^= x >> 16;
+  return x;
+}
+
+__device__ __forceinline__ uint32_t noise_key(uint32_t lo, uint32_t hi, uint32_t index) {
+  const uint32_t key = fmix(lo ^ fmix(hi + 0x9E3779B9u));
+  return fmix(key ^ fmix(index + 0x7F4A7C15u));
+}
+
+__device__ __forceinline__ float uniform_noise(uint32_t key, uint32_t v) {
+  uint32_t x = fmix(key + v * 0x9E3779B1u);
+  x = fmix(x ^ key);
+  return (static_cast<float>(x >> 9) + 0.5f) * (1.0f / 8388608.0f);
+}
+
+// float32 -> unsigned key with the same order
+__device__ __forceinline__ uint32_t order_key(float f) {
+  const uint32_t b = __float_as_uint(f);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+struct Best {
+  float val;
+  int idx;
+};
+
+__device__ __forceinline__ Best better(Best a, Best b) {
+  if (b.idx < 0) return a;
+  if (a.idx < 0) return b;
+  if (b.val > a.val || (b.val == a.val && b.idx < a.idx)) return b;
+  return a;
+}
+
+__device__ Best block_best(Best mine, Best* scratch) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    Best other;
+    other.val = __shfl_xor(mine.val, o, kWave);
+    other.idx = __shfl_xor(mine.idx, o, kWave);
+    mine = better(mine, other);
+  }
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = mine;
+  __syncthreads();
+  Best total = scratch[0];
+  for (int w = 1; w < kThreads / kWave; ++w) total = better(total, scratch[w]);
+  return total;
+}
+
+__device__ float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = scratch[0];
+  for (int w = 1; w < kThreads / kWave; ++w) total = fmaxf(total, scratch[w]);
+  return total;
+}
+
+__global__ __launch_bounds__(kThreads) void argmax_kernel(int32_t* __restrict__ out,
+                                                          const float* __restrict__ logits, int V,
+                                                          int64_t row_stride) {
+  __shared__ Best scratch[kThreads / kWave];
+  const float* row = logits + static_cast<int64_t>(blockIdx.x) * row_stride;
+  Best mine{-INFINITY, -1};
+  for (int v = threadIdx.x; v < V; v += kThreads) mine = better(mine, Best{row[v], v});
+  const Best total = block_best(mine, scratch);
+  if (threadIdx.x == 0) out[blockIdx.x] = total.idx < 0 ? 0 : total.idx;
+}
+
+__global__ __launch_bounds__(kThreads) void sample_kernel(
+    int32_t* __restrict__ out, const float* __restrict__ logits, int V, int64_t row_stride,
+    const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
+    const float* __restrict__ top_p, const uint32_t* __restrict__ seed_lo,
+    const uint32_t* __restrict__ seed_hi, const uint32_t* __restrict__ index) {
+  __shared__ Best best_scratch[kThreads / kWave];
+  __shared__ float f_scratch[kThreads / kWave];
+  const int s = blockIdx.x;
+  const float* row = logits + static_cast<int64_t>(s) * row_stride;
+  const float temp = temperature[s];
+
+  if (temp < kGreedyEps) {
+    Best mine{-INFINITY, -1};
+    for (int v = threadIdx.x; v < V; v += kThreads) mine = better(mine, Best{row[v], v});
+    const Best total = block_best(mine, best_scratch);
+    if (threadIdx.x == 0) out[s] = total.idx < 0 ? 0 : total.idx;
+    return;
+  }
+  const float inv_t = 1.0f / temp;
+  int k = top_k[s];
+  if (k <= 0 || k > V) k = V;
+  const float p_keep = top_p[s];
+
+  // threshold key: entries with order_key(z) >= keep_key stay
+  uint32_t keep_key = 0u;
+  if (k < V) {
+    // the k-th largest value: the largest key with at least k entries at or above it
+    uint32_t lo = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t cand = lo | (1u << bit);
+      float cnt = 0.f;
+      for (int v = threadIdx.x; v < V; v += kThreads)
+        cnt += (order_key(row[v] * inv_t) >= cand) ? 1.f : 0.f;
+      const float total = block_sum(cnt, f_scratch);
+      if (total >= static_cast<float>(k)) lo = cand;
+    }
+    keep_key = lo;
+  }
+  if (p_keep < 1.0f) {
+    float zmax = -INFINITY;
+    for (int v = threadIdx.x; v < V; v += kThreads) zmax = fmaxf(zmax, row[v] * inv_t);
+    zmax = block_max(zmax, f_scratch);
+    const uint32_t max_key = order_key(zmax);
+    float den = 0.f;
+    for (int v = threadIdx.x; v < V; v += kThreads) {
+      const float z = row[v] * inv_t;
+      if (order_key(z) >= keep_key) den += expf(z - zmax);
+    }
+    den = block_sum(den, f_scratch);
+    const float limit = (1.0f - p_keep) * den;
+    // the largest key whose strictly-smaller kept entries weigh at most `limit`
+    uint32_t lo = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t cand = lo | (1u << bit);
+      float mass = 0.f;
+      for (int v = threadIdx.x; v < V; v += kThreads) {
+        const float z = row[v] * inv_t;
+        const uint32_t key = order_key(z);
+        if (key >= keep_key && key < cand) mass += expf(z - zmax);
+      }
+      mass = block_sum(mass, f_scratch);
+      if (mass <= limit) lo = cand;
+    }
+    if (lo > max_key) lo = max_key;  // the largest entry is never dropped
+    if (lo > keep_key) keep_key = lo;
+  }
+
+  const uint32_t key = noise_key(seed_lo[s], seed_hi[s], index[s]);
+  Best mine{-INFINITY, -1};
+  for (int v = threadIdx.x; v < V; v += kThreads) {
+    const float z = row[v] * inv_t;
+    if (order_key(z) < keep_key) continue;
+    const float e = -logf(uniform_noise(key, static_cast<uint32_t>(v)));
+    mine = better(mine, Best{z - logf(e), v});
+  }
+  const Best total = block_best(mine, best_scratch);
+  if (threadIdx.x == 0) out[s] = total.idx < 0 ? 0 : total.idx;
+}
+
+}  // namespace
+
+extern "C" int kvc_argmax(int32_t* out, const float* logits, int S_, int V, int64_t row_stride,
+                          kvc_stream stream) {
+  if (S_ < 0 || V <= 0 || row_stride < V) return kvc_fail("kvc_argmax: bad sizes");
+  if (S_ == 0) return 0;
+  hipLaunchKernelGGL(argmax_kernel, dim3(S_), dim3(kThreads), 0,
+                     reinterpret_cast<hipStream_t>(stream), out, logits, V, row_stride);
+  return kvc_check_launch("kvc_argmax");
+}
+
+extern "C" int kvc_sample(int32_t* out, const float* logits, int S_, int V, int64_t row_stride,
+                          const float* temperature, const int32_t* top_k, const float* top_p,
+                          const uint32_t* seed_lo, const uint32_t* seed_hi, const uint32_t* index,
+                          kvc_stream stream) {
+  if (S_ < 0 || V <= 0 || row_stride < V) return kvc_fail("kvc_sample: bad sizes");
+  if (S_ == 0) return 0;
+  hipLaunchKernelGGL(sample_kernel, dim3(S_), dim3(kThreads), 0,
+                     reinterpret_cast<hipStream_t>(stream), out, logits, V, row_stride,
+                     temperature, top_k, top_p, seed_lo, seed_hi, index);
+  return kvc_check_launch("kvc_sample");
+}

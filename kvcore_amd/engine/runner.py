@@ -1,0 +1,292 @@
+"""The step function: one batch of (request, its next tokens) through the model, from
+the cache, to logits at the wanted places.
+
+Reference: kvcore/model/model_runner.py:208-306 (``execute_model``: update states,
+flatten, build metadata, forward, logits at selected rows) with kvcore/model/
+input_batch.py and kvcore/kv/block_table.py.  Differences that matter:
+
+* a request keeps its slot (its block-table row) for life, so nothing is condensed or
+  moved between steps (input_batch.py:202-223 moves rows);
+* one block table per cache group serves all planes of the group, and the slot of a
+  token is computed inside the kernels from table and position (block_table.py:196-228
+  builds a slot mapping per layer in Python);
+* one packed int32 upload per step carries every index array and the block-table
+  changes (model_runner.py:475-509 uploads seven tensors and 3 per layer);
+* the caller says where logits are wanted; the reference takes them only at the last
+  token of a request whose known tokens are all computed (model_runner.py:461-464).
+"""
+
+from __future__ import annotations
+
+import json
+from dataclasses import dataclass, field
+from pathlib import Path
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from kvcore_amd.config.model_config import read_config_json
+from kvcore_amd.models.decoder import DecoderModel
+from kvcore_amd.ops import library as ops
+from kvcore_amd.registry import resolve_architecture
+
+from .context import CacheGroupView, StepBuffers, StepContext
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: ``tokens`` go to positions ``start ..``;
+    ``pages[g]`` is the request's page list in cache group ``g`` (covering at least
+    ``start + len(tokens)`` tokens); ``want`` lists indices into ``tokens`` whose logits
+    are asked for."""
+
+    request_id: str
+    slot: int
+    start: int
+    tokens: Sequence[int]
+    pages: Sequence[Sequence[int]]
+    want: Sequence[int] = ()
+    released: Sequence[int] | None = None  # per group: leading page entries that are null
+
+
+@dataclass
+class StepOutput:
+    """``logits`` is float32 ``[S, V]`` on the device (None when nothing was wanted);
+    row ``i`` belongs to ``owners[i] = (index of the entry in the step, position)``."""
+
+    request_ids: list[str]
+    logits: torch.Tensor | None
+    owners: list[tuple[int, int]] = field(default_factory=list)
+    num_tokens: int = 0
+
+
+def build_model(model_dir: str | Path, dtype: torch.dtype, device: str | torch.device,
+                *, load_format: str = "safetensors", seed: int = 0, strict: bool = True,
+                config_override: dict | None = None) -> DecoderModel:
+    """config.json -> registry -> spec -> model with weights.  ``load_format="random"``
+    fills the parameters from ``seed`` instead of reading weight files."""
+    from kvcore_amd.weights.loader import init_random_weights, load_weights
+
+    config = config_override if config_override is not None else read_config_json(model_dir)
+    arch = resolve_architecture(config)
+    typed = arch.parse_config(config)
+    spec = arch.build_spec(typed)
+    model = DecoderModel(spec, dtype, device)
+    model.typed_config = typed
+    if load_format == "random":
+        init_random_weights(model, seed)
+    else:
+        load_weights(model, model_dir, strict=strict)
+    return model
+
+
+class ModelRunner:
+    """Owns the device side of the cache (planes, block tables, state arrays), the step
+    buffers and the model; runs steps."""
+
+    def __init__(self, model: DecoderModel, *, page_size: int, num_pages: int | Sequence[int],
+                 max_num_seqs: int, max_num_tokens: int, max_model_len: int) -> None:
+        ops.load()  # fail here, loudly, if the kernels are not there
+        if model.device.type != "cuda":
+            raise RuntimeError("kvcore_amd runs on a GPU only; there is no CPU path")
+        self.model = model
+        self.device = model.device
+        self.dtype = model.dtype
+        self.page_size = page_size
+        self.max_num_seqs = max_num_seqs
+        self.max_num_tokens = max_num_tokens
+        self.max_model_len = max_model_len
+        self.max_pages_per_seq = -(-max_model_len // page_size)
+        n_groups = len(model.cache_groups)
+        self.num_pages = [num_pages] * n_groups if isinstance(num_pages, int) else list(num_pages)
+        if len(self.num_pages) != n_groups:
+            raise ValueError("num_pages must give one count per cache group")
+
+        self.groups: list[CacheGroupView] = []
+        for gs, pages in zip(model.cache_groups, self.num_pages):
+            kv = torch.empty((gs.num_planes, 2, pages, gs.need.num_kv_heads, page_size,
+                              gs.need.head_dim), dtype=self.dtype, device=self.device)
+            table = torch.zeros((max_num_seqs, self.max_pages_per_seq), dtype=torch.int32,
+                                device=self.device)
+            self.groups.append(CacheGroupView(kv, table, page_size, gs.need.window))
+        self.states = [
+            torch.zeros((max_num_seqs, *sa.need.shape), dtype=sa.need.dtype, device=self.device)
+            for sa in model.state_arrays
+        ]
+        self.buffers = StepBuffers(self.device)
+
+        # host mirror of what each slot's table rows hold: (request id, entries synced,
+        # leading entries nulled) per group
+        self._slot_owner: list[str | None] = [None] * max_num_seqs
+        self._slot_synced = [[0] * n_groups for _ in range(max_num_seqs)]
+        self._slot_released = [[0] * n_groups for _ in range(max_num_seqs)]
+
+        # packed per-step metadata: fixed layout, one upload
+        T, R = max_num_tokens, max_num_seqs
+        self._upd_cap = 2 * (T + R)
+        sections = [("token_ids", T), ("positions", T), ("token_req", T), ("logit_rows", T),
+                    ("q_start", R + 1), ("seq_lens", R), ("slots", R)]
+        self._off: dict[str, tuple[int, int]] = {}
+        cursor = 0
+        for name, n in sections:
+            self._off[name] = (cursor, n)
+            cursor += n
+        self._upd_off = cursor
+        total = cursor + 3 * self._upd_cap * max(n_groups, 1)
+        self._meta_host = torch.empty(total, dtype=torch.int32, pin_memory=True)
+        self._meta_np = self._meta_host.numpy()
+        self._meta_dev = torch.zeros(total, dtype=torch.int32, device=self.device)
+        self._dev = {name: self._meta_dev[o:o + n] for name, (o, n) in self._off.items()}
+        self._np = {name: self._meta_np[o:o + n] for name, (o, n) in self._off.items()}
+        self._copy_done = torch.cuda.Event()
+        self._copy_pending = False
+
+    # -------------------------------------------------------------------- bookkeeping
+    def forget(self, slot: int) -> None:
+        """A request left its slot.  The next owner's pages are synced from scratch."""
+        self._slot_owner[slot] = None
+
+    def fill_cache(self, value: float) -> None:
+        """Overwrite every cache plane (tests fill with NaN so that a read outside a
+        request's own slots shows in the logits)."""
+        for g in self.groups:
+            g.kv.fill_(value)
+
+    def cache_bytes_per_page(self) -> int:
+        return sum(gs.num_planes * 2 * gs.need.num_kv_heads * self.page_size * gs.need.head_dim
+                   for gs in self.model.cache_groups) * torch.empty((), dtype=self.dtype).element_size()
+
+    def _table_updates(self, entries: Sequence[StepEntry]) -> list[list[int]]:
+        """Per group, flat triples (slot, index, page) that bring the device tables up to
+        the entries' page lists."""
+        n_groups = len(self.groups)
+        out: list[list[int]] = [[] for _ in range(n_groups)]
+        for e in entries:
+            slot = e.slot
+            fresh = self._slot_owner[slot] != e.request_id
+            if fresh:
+                self._slot_owner[slot] = e.request_id
+                self._slot_synced[slot] = [0] * n_groups
+                self._slot_released[slot] = [0] * n_groups
+            for g in range(n_groups):
+                pages = e.pages[g]
+                have = self._slot_synced[slot][g]
+                if len(pages) > have:
+                    upd = out[g]
+                    for i in range(have, len(pages)):
+                        upd.extend((slot, i, pages[i]))
+                    self._slot_synced[slot][g] = len(pages)
+                if e.released is not None:
+                    done = self._slot_released[slot][g]
+                    if e.released[g] > done:
+                        upd = out[g]
+                        for i in range(done, e.released[g]):
+                            upd.extend((slot, i, 0))
+                        self._slot_released[slot][g] = e.released[g]
+        return out
+
+    # --------------------------------------------------------------------------- step
+    def step(self, entries: Sequence[StepEntry]) -> StepOutput:
+        """Run exactly the tokens given, as one batch, from the cache earlier steps left.
+        Keys and values of these tokens are written to their pages first and read back
+        from there, so what a position computes does not depend on how its request was
+        cut into steps."""
+        R = len(entries)
+        if R == 0:
+            return StepOutput([], None)
+        if R > self.max_num_seqs:
+            raise ValueError(f"{R} requests in a step exceed max_num_seqs={self.max_num_seqs}")
+        vocab = self.model.spec.vocab_size
+        npv = self._np
+        t = 0
+        owners: list[tuple[int, int]] = []
+        n_rows = 0
+        q_lens: list[int] = []
+        seq_lens: list[int] = []
+        seen_slots: set[int] = set()
+        if self._copy_pending:
+            self._copy_done.synchronize()
+            self._copy_pending = False
+        for r, e in enumerate(entries):
+            n = len(e.tokens)
+            if n == 0:
+                raise ValueError(f"request {e.request_id!r}: a step entry needs at least one token")
+            end = e.start + n
+            if e.start < 0 or end > self.max_model_len:
+                raise ValueError(f"request {e.request_id!r}: positions {e.start}..{end - 1} exceed "
+                                 f"max_model_len={self.max_model_len}")
+            if t + n > self.max_num_tokens:
+                raise ValueError(f"step exceeds max_num_tokens={self.max_num_tokens}")
+            if not 0 <= e.slot < self.max_num_seqs or e.slot in seen_slots:
+                raise ValueError(f"request {e.request_id!r}: slot {e.slot} is invalid or used twice")
+            seen_slots.add(e.slot)
+            for g, grp in enumerate(self.groups):
+                if len(e.pages[g]) * self.page_size < end:
+                    raise ValueError(f"request {e.request_id!r}: {len(e.pages[g])} pages do not hold "
+                                     f"{end} tokens")
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            if toks.min() < 0 or toks.max() >= vocab:
+                raise ValueError(f"request {e.request_id!r}: token id outside [0, {vocab})")
+            npv["token_ids"][t:t + n] = toks
+            npv["positions"][t:t + n] = np.arange(e.start, end, dtype=np.int32)
+            npv["token_req"][t:t + n] = r
+            npv["q_start"][r] = t
+            npv["seq_lens"][r] = end
+            npv["slots"][r] = e.slot
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise ValueError(f"request {e.request_id!r}: wanted index {w} outside its {n} tokens")
+                npv["logit_rows"][n_rows] = t + w
+                owners.append((r, e.start + w))
+                n_rows += 1
+            q_lens.append(n)
+            seq_lens.append(end)
+            t += n
+        T = t
+        npv["q_start"][R] = T
+
+        updates = self._table_updates(entries)
+        upd_counts = []
+        cursor = self._upd_off
+        for g, upd in enumerate(updates):
+            count = len(upd) // 3
+            if count > self._upd_cap:
+                raise RuntimeError("block-table update overflow")  # cannot happen: bounded by pages per step
+            if count:
+                self._meta_np[cursor:cursor + 3 * count] = upd
+            upd_counts.append((cursor, count))
+            cursor += 3 * count
+        self._meta_dev[:cursor].copy_(self._meta_host[:cursor], non_blocking=True)
+        self._copy_done.record()
+        self._copy_pending = True
+        for g, (off, count) in enumerate(upd_counts):
+            if count:
+                ops.table_update(self.groups[g].table, self._meta_dev[off:off + 3 * count], count)
+
+        ctx = StepContext(
+            num_tokens=T, num_reqs=R,
+            token_ids=self._dev["token_ids"], positions=self._dev["positions"],
+            token_req=self._dev["token_req"], q_start=self._dev["q_start"],
+            seq_lens=self._dev["seq_lens"], slots=self._dev["slots"],
+            groups=self.groups, states=self.states, buffers=self.buffers,
+            dtype=self.dtype, device=self.device,
+            host_query_lens=q_lens, host_seq_lens=seq_lens,
+            max_query_len=max(q_lens), max_seq_len=max(seq_lens),
+        )
+        hidden = self.model.forward(ctx)
+        logits = None
+        if n_rows:
+            logits = self.model.compute_logits(ctx, hidden, self._dev["logit_rows"], n_rows)
+        return StepOutput([e.request_id for e in entries], logits, owners, T)
+
+
+def describe_model(model: DecoderModel) -> str:
+    spec = model.spec
+    return json.dumps({
+        "layers": len(spec.layers), "schedule": len(spec.resolved_schedule()),
+        "hidden": spec.hidden_size, "vocab": spec.vocab_size,
+        "cache_groups": [(g.need.num_kv_heads, g.need.head_dim, g.need.window, g.num_planes)
+                         for g in model.cache_groups],
+        "param_bytes": model.num_param_bytes(),
+    })

@@ -1,0 +1,180 @@
+"""The generic decoder: builds the parts a ``ModelSpec`` names, owns their parameters,
+runs the schedule.
+
+Reference: kvcore/model/models/llama3.py:145-247 (embedding, layer loop, final norm,
+head).  Which architecture this is, is decided wholly by the spec.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from kvcore_amd.engine.context import LayerCall, StepContext
+from kvcore_amd.ops import library as ops
+from kvcore_amd.parts import base as parts
+from kvcore_amd.parts.base import CacheNeed, ParamSpec, Part, Runtime, StateNeed
+from kvcore_amd.parts.embedding import OutputHead, TokenEmbedding
+
+from .spec import ModelSpec
+
+
+@dataclass(frozen=True)
+class CacheGroupSpec:
+    """Entries of the schedule whose mixers need the same kind of paged memory share a
+    group: one page pool, one block table per request, ``num_planes`` cache planes."""
+
+    need: CacheNeed
+    num_planes: int
+
+
+@dataclass(frozen=True)
+class StateArraySpec:
+    need: StateNeed
+
+
+@dataclass
+class BoundParam:
+    name: str  # full parameter name
+    prefix: str  # checkpoint prefix of the owning part
+    spec: ParamSpec
+    tensor: torch.Tensor
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device: torch.device | str) -> None:
+        self.spec = spec
+        self.runtime = Runtime(dtype=dtype, device=torch.device(device))
+        self.dtype = dtype
+        self.device = self.runtime.device
+
+        self.positions = [parts.POSITION_ENCODINGS.build(p) for p in spec.positions]
+        self.embed = TokenEmbedding(vocab_size=spec.vocab_size, hidden_size=spec.hidden_size)
+        self.head = OutputHead(vocab_size=spec.vocab_size, hidden_size=spec.hidden_size,
+                               tied=spec.tie_word_embeddings)
+        self.final_norm = parts.NORMS.build(spec.final_norm)
+        self.blocks: list[parts.Block] = []
+        for layer in spec.layers:
+            position = None if layer.position is None else self.positions[layer.position]
+            mixer = parts.MIXERS.build(layer.mixer, position=position)
+            ffn = parts.FEED_FORWARDS.build(layer.ffn)
+            norms = {name: parts.NORMS.build(ns) for name, ns in layer.norms.items()}
+            self.blocks.append(parts.BLOCKS.build(layer.block, mixer=mixer, ffn=ffn, norms=norms))
+
+        self._owned: list[tuple[str, Part]] = [(spec.embed_prefix, self.embed),
+                                               (spec.final_norm_prefix, self.final_norm),
+                                               (spec.head_prefix, self.head)]
+        for layer, block in zip(spec.layers, self.blocks):
+            for sub, part in block.children().items():
+                self._owned.append((f"{layer.prefix}.{sub}", part))
+        for _, part in self._owned:
+            part.setup(self.runtime)
+        for pe in self.positions:
+            pe.setup(self.runtime)
+
+        self._plan_caches()
+        self.params: dict[str, BoundParam] = {}
+        self._allocate_params()
+
+    # ---------------------------------------------------------------- cache planning
+    def _plan_caches(self) -> None:
+        schedule = self.spec.resolved_schedule()
+        group_of: dict[CacheNeed, int] = {}
+        planes: list[int] = []
+        needs: list[CacheNeed] = []
+        states: list[StateArraySpec] = []
+        calls: list[LayerCall] = []
+        for e, entry in enumerate(schedule):
+            if not 0 <= entry.layer < len(self.blocks):
+                raise ValueError(f"schedule entry {e} names layer {entry.layer}, which does not exist")
+            mixer = self.blocks[entry.layer].mixer
+            need = mixer.cache_need()
+            g = plane = None
+            write = True
+            if need is not None:
+                if entry.cache_from is not None:
+                    if not 0 <= entry.cache_from < e:
+                        raise ValueError(f"schedule entry {e}: cache_from must name an earlier entry")
+                    src = calls[entry.cache_from]
+                    if src.group_index is None or needs[src.group_index] != need:
+                        raise ValueError(f"schedule entry {e}: entry {entry.cache_from} has no cache "
+                                         "of the shape this layer reads")
+                    g, plane, write = src.group_index, src.cache_index, False
+                else:
+                    if need not in group_of:
+                        group_of[need] = len(needs)
+                        needs.append(need)
+                        planes.append(0)
+                    g = group_of[need]
+                    plane = planes[g]
+                    planes[g] += 1
+            state_need = mixer.state_need()
+            state_index = None
+            if state_need is not None:
+                state_index = len(states)
+                states.append(StateArraySpec(state_need))
+            calls.append(LayerCall(e, entry.layer, g, plane, write, state_index))
+        self.calls = calls
+        self.cache_groups = [CacheGroupSpec(n, c) for n, c in zip(needs, planes)]
+        self.state_arrays = states
+
+    # -------------------------------------------------------------------- parameters
+    def _allocate_params(self) -> None:
+        kinds = {"matrix": self.dtype, "vector": torch.float32, "table": torch.int32}
+        for prefix, part in self._owned:
+            local: dict[str, torch.Tensor] = {}
+            for ps in part.param_specs():
+                t = torch.empty(ps.shape, dtype=kinds[ps.kind], device=self.device)
+                full = f"{prefix}.{ps.name}"
+                if full in self.params:
+                    raise ValueError(f"parameter {full} is declared twice")
+                self.params[full] = BoundParam(full, prefix, ps, t)
+                local[ps.name] = t
+            part.bind(local)
+        if self.spec.tie_word_embeddings:
+            self.head.bind({"weight": self.embed.params["weight"]})
+
+    def checkpoint_map(self) -> dict[str, tuple[BoundParam, int, int]]:
+        """Checkpoint tensor name -> (parameter, first row, rows)."""
+        out: dict[str, tuple[BoundParam, int, int]] = {}
+        for bp in self.params.values():
+            for src in bp.spec.resolved_sources():
+                out[f"{bp.prefix}.{src.name}"] = (bp, src.row, src.rows)
+        return out
+
+    def optional_checkpoint_names(self) -> set[str]:
+        """Names a file may hold that are not read: a tied head's own matrix
+        (reference: kvcore/model/model_utils.py:51-53)."""
+        if self.spec.tie_word_embeddings:
+            return {f"{self.spec.head_prefix}.weight"}
+        return set()
+
+    def num_param_bytes(self) -> int:
+        return sum(bp.tensor.numel() * bp.tensor.element_size() for bp in self.params.values())
+
+    # ----------------------------------------------------------------------- forward
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        """Normalised hidden rows ``[T, H]`` in the model dtype for the batch in ``ctx``."""
+        H = self.spec.hidden_size
+        residual = ctx.buf("residual", H, torch.float32)
+        self.embed.forward(residual, ctx.token_ids[: ctx.num_tokens])
+        for pe in self.positions:
+            pe.prepare(ctx)
+            pe.embed(residual, ctx)
+        delta = None
+        for call in self.calls:
+            delta = self.blocks[call.layer_index].forward(delta, residual, ctx, call)
+        hidden = ctx.buf("final_hidden", H)
+        self.final_norm.forward_fused(hidden, residual, delta)
+        return hidden
+
+    def compute_logits(self, ctx: StepContext, hidden: torch.Tensor, rows: torch.Tensor,
+                       num_rows: int) -> torch.Tensor:
+        """float32 ``[S, V]`` at the flattened token indices ``rows[:S]``."""
+        H, V = self.spec.hidden_size, self.spec.vocab_size
+        picked = ctx.buffers.get("head_rows", num_rows, H, self.dtype)
+        ops.gather_rows(picked, hidden, rows[:num_rows])
+        logits = ctx.buffers.get("logits", num_rows, V, torch.float32)
+        self.head.forward(logits, picked, ctx)
+        return logits

@@ -1,0 +1,54 @@
+"""A model as data: layers chosen part by part, and the order in which they run."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any
+
+from kvcore_amd.parts.base import PartSpec
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One layer's parts.  ``position`` indexes ``ModelSpec.positions`` (None: the mixer
+    gets no position encoding); ``norms`` maps the block's norm names to norm specs;
+    ``prefix`` is the layer's checkpoint prefix."""
+
+    prefix: str
+    mixer: PartSpec
+    ffn: PartSpec
+    norms: dict[str, PartSpec]
+    block: PartSpec = field(default_factory=lambda: PartSpec("prenorm"))
+    position: int | None = None
+
+
+@dataclass(frozen=True)
+class ScheduleEntry:
+    """Run ``layer``.  ``cache_from`` names an earlier schedule entry (by its index in the
+    schedule) whose cache this entry reads instead of writing its own."""
+
+    layer: int
+    cache_from: int | None = None
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    vocab_size: int
+    hidden_size: int
+    max_position_embeddings: int
+    layers: tuple[LayerSpec, ...]
+    final_norm: PartSpec
+    positions: tuple[PartSpec, ...] = ()
+    schedule: tuple[ScheduleEntry, ...] = ()
+    tie_word_embeddings: bool = False
+    eos_token_ids: tuple[int, ...] = ()
+    embed_prefix: str = "model.embed_tokens"
+    final_norm_prefix: str = "model.norm"
+    head_prefix: str = "lm_head"
+    # checkpoint names that may be present and are not read (reference:
+    # kvcore/model/model_utils.py:49-50 skips rotary_emb.inv_freq buffers)
+    ignored_suffixes: tuple[str, ...] = ("rotary_emb.inv_freq",)
+    extra: dict[str, Any] = field(default_factory=dict)
+
+    def resolved_schedule(self) -> tuple[ScheduleEntry, ...]:
+        return self.schedule or tuple(ScheduleEntry(i) for i in range(len(self.layers)))

@@ -1,0 +1,295 @@
+"""Python face of the gfx950 kernel library: loads it, checks operands on the host,
+launches on torch's current stream.
+
+There is no other compute path.  If the library cannot be loaded or built, the first
+use raises; nothing falls back to the CPU or to torch's operators (library matrix
+products for bfloat16 excepted, which is where the reference uses a library too:
+``nn.Linear`` at kvcore/model/layer/linear.py:6-11).
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_void_p
+
+import torch
+
+from . import build as _build
+
+_LIB: ctypes.CDLL | None = None
+_LIB_PATH: str | None = None
+
+DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    """The kernel library refused its arguments or could not launch."""
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    P, I, L, F = c_void_p, c_int, c_int64, c_float
+    sigs = {
+        "kvc_embed": [P, P, P, I, I, I, I, P],
+        "kvc_add_rmsnorm": [P, P, P, P, F, I, I, I, P],
+        "kvc_rmsnorm": [P, P, P, F, I, I, L, L, I, P],
+        "kvc_residual_add": [P, P, I, I, I, P],
+        "kvc_silu_mul": [P, P, I, I, I, P],
+        "kvc_gather_rows": [P, P, P, I, I, I, I, P],
+        "kvc_to_float": [P, P, L, I, P],
+        "kvc_rope_table": [P, P, P, P, I, I, P],
+        "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
+        "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
+        "kvc_table_update": [P, I, I, P, I, P],
+        "kvc_argmax": [P, P, I, I, L, P],
+        "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P],
+    }
+    for name, argtypes in sigs.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+    lib.kvc_last_error.restype = ctypes.c_char_p
+    lib.kvc_last_error.argtypes = []
+    lib.kvc_version.restype = c_int
+
+
+def load(build_if_missing: bool = True) -> ctypes.CDLL:
+    """The loaded library; built first when no matching build is found."""
+    global _LIB, _LIB_PATH
+    if _LIB is not None:
+        return _LIB
+    path = _build.find_library()
+    if path is None:
+        if not build_if_missing:
+            raise KernelError("kvcore_amd: the gfx950 kernel library is not built")
+        path = _build.build()
+    try:
+        lib = ctypes.CDLL(str(path))
+    except OSError as exc:
+        raise KernelError(f"kvcore_amd: cannot load the kernel library {path}: {exc}") from exc
+    _declare(lib)
+    _LIB, _LIB_PATH = lib, str(path)
+    return lib
+
+
+def library_path() -> str | None:
+    return _LIB_PATH
+
+
+def _check(code: int, name: str) -> None:
+    if code != 0:
+        msg = load().kvc_last_error().decode("utf-8", "replace")
+        raise KernelError(f"{name} failed ({code}): {msg}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, name: str, dtype: torch.dtype | None = None) -> int:
+    if not t.is_cuda:
+        raise KernelError(f"{name} must be a GPU tensor (this engine has no CPU path)")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    return t.data_ptr()
+
+
+def _code(t: torch.Tensor, name: str) -> int:
+    try:
+        return DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"{name}: unsupported dtype {t.dtype}") from None
+
+
+# ------------------------------------------------------------------------ wrappers
+def embed(residual: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+    T, H = residual.shape
+    V = table.shape[0]
+    if table.shape[1] != H or ids.numel() != T:
+        raise KernelError("embed: shapes do not match")
+    _check(load().kvc_embed(_dev(residual, "residual", torch.float32), _dev(table, "table"),
+                            _dev(ids, "ids", torch.int32), T, H, V, _code(table, "table"), _stream()),
+           "kvc_embed")
+
+
+def add_rmsnorm(out: torch.Tensor, residual: torch.Tensor, delta: torch.Tensor | None,
+                weight: torch.Tensor, eps: float) -> None:
+    T, H = residual.shape
+    if out.shape != (T, H) or weight.shape != (H,) or (delta is not None and delta.shape != (T, H)):
+        raise KernelError("add_rmsnorm: shapes do not match")
+    if delta is not None and delta.dtype != out.dtype:
+        raise KernelError("add_rmsnorm: delta and out must share a dtype")
+    _check(load().kvc_add_rmsnorm(_dev(out, "out"), _dev(residual, "residual", torch.float32),
+                                  None if delta is None else _dev(delta, "delta"),
+                                  _dev(weight, "weight", torch.float32), float(eps), T, H,
+                                  _code(out, "out"), _stream()), "kvc_add_rmsnorm")
+
+
+def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+    """Rows of ``x`` (last dim contiguous, any row stride) normalised into ``out``."""
+    if x.dim() != 2 or out.shape != x.shape or x.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("rmsnorm: expects 2-D tensors with a contiguous last dim")
+    if x.dtype != out.dtype or not x.is_cuda or not out.is_cuda:
+        raise KernelError("rmsnorm: x and out must be GPU tensors of one dtype")
+    T, H = x.shape
+    if weight.shape != (H,):
+        raise KernelError("rmsnorm: weight shape")
+    _check(load().kvc_rmsnorm(out.data_ptr(), x.data_ptr(), _dev(weight, "weight", torch.float32),
+                              float(eps), T, H, x.stride(0), out.stride(0), _code(x, "x"), _stream()),
+           "kvc_rmsnorm")
+
+
+def residual_add(residual: torch.Tensor, delta: torch.Tensor) -> None:
+    T, H = residual.shape
+    if delta.shape != (T, H):
+        raise KernelError("residual_add: shapes do not match")
+    _check(load().kvc_residual_add(_dev(residual, "residual", torch.float32), _dev(delta, "delta"),
+                                   T, H, _code(delta, "delta"), _stream()), "kvc_residual_add")
+
+
+def silu_mul(out: torch.Tensor, gate_up: torch.Tensor) -> None:
+    T, I2 = gate_up.shape
+    if I2 % 2 or out.shape != (T, I2 // 2) or out.dtype != gate_up.dtype:
+        raise KernelError("silu_mul: shapes or dtypes do not match")
+    _check(load().kvc_silu_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), T, I2 // 2,
+                               _code(out, "out"), _stream()), "kvc_silu_mul")
+
+
+def gather_rows(out: torch.Tensor, src: torch.Tensor, rows: torch.Tensor) -> None:
+    S, H = out.shape
+    if src.shape[1] != H or rows.numel() != S:
+        raise KernelError("gather_rows: shapes do not match")
+    _check(load().kvc_gather_rows(_dev(out, "out"), _dev(src, "src"), _dev(rows, "rows", torch.int32),
+                                  S, H, _code(src, "src"), _code(out, "out"), _stream()),
+           "kvc_gather_rows")
+
+
+def to_float(out: torch.Tensor, src: torch.Tensor) -> None:
+    if out.numel() != src.numel():
+        raise KernelError("to_float: sizes do not match")
+    _check(load().kvc_to_float(_dev(out, "out", torch.float32), _dev(src, "src"), src.numel(),
+                               _code(src, "src"), _stream()), "kvc_to_float")
+
+
+def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+               inv_freq: torch.Tensor) -> None:
+    T, half = cos.shape
+    if sin.shape != (T, half) or positions.numel() < T or inv_freq.numel() != half:
+        raise KernelError("rope_table: shapes do not match")
+    _check(load().kvc_rope_table(_dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32),
+                                 _dev(positions, "positions", torch.int32),
+                                 _dev(inv_freq, "inv_freq", torch.float32), T, half, _stream()),
+           "kvc_rope_table")
+
+
+def rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  cos: torch.Tensor, sin: torch.Tensor, *, rot_dim: int, interleaved: bool,
+                  positions: torch.Tensor, token_req: torch.Tensor, slots: torch.Tensor,
+                  table: torch.Tensor, nh: int, nkv: int, d: int, write_kv: bool = True) -> None:
+    """``k_cache``/``v_cache`` are ``[pages, nkv, page_size, d]`` of the dtype of ``qkv``."""
+    T = qkv.shape[0]
+    if qkv.shape != (T, (nh + 2 * nkv) * d):
+        raise KernelError(f"rope_kv_write: qkv shape {tuple(qkv.shape)} does not fit heads")
+    num_pages, ckv, page_size, cd = k_cache.shape
+    if (ckv, cd) != (nkv, d) or v_cache.shape != k_cache.shape:
+        raise KernelError("rope_kv_write: cache shape does not fit heads")
+    if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
+        raise KernelError("rope_kv_write: cache dtype differs from qkv")
+    if cos.shape[0] < T or cos.shape[1] != rot_dim // 2 or sin.shape != cos.shape:
+        raise KernelError("rope_kv_write: rotary tables do not fit")
+    if positions.numel() < T or token_req.numel() < T:
+        raise KernelError("rope_kv_write: per-token arrays too short")
+    _check(load().kvc_rope_kv_write(
+        _dev(qkv, "qkv"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
+        _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), rot_dim, int(interleaved),
+        _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
+        _dev(slots, "slots", torch.int32), _dev(table, "table", torch.int32), table.shape[1],
+        T, nh, nkv, d, page_size, num_pages, int(write_kv), _code(qkv, "qkv"), _stream()),
+        "kvc_rope_kv_write")
+
+
+def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    *, table: torch.Tensor, positions: torch.Tensor, token_req: torch.Tensor,
+                    slots: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
+                    window: int = 0) -> None:
+    """``q`` is a ``[T, >= nh*d]`` view whose rows hold the query heads first."""
+    T = out.shape[0]
+    if out.shape != (T, nh * d) or not out.is_contiguous():
+        raise KernelError("paged_attention: out must be contiguous [T, nh*d]")
+    if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or q.dtype != out.dtype:
+        raise KernelError("paged_attention: q does not fit")
+    num_pages, ckv, page_size, cd = k_cache.shape
+    if (ckv, cd) != (nkv, d) or v_cache.shape != k_cache.shape or k_cache.dtype != out.dtype:
+        raise KernelError("paged_attention: cache does not fit heads or dtype")
+    if positions.numel() < T or token_req.numel() < T:
+        raise KernelError("paged_attention: per-token arrays too short")
+    _check(load().kvc_paged_attention(
+        out.data_ptr(), q.data_ptr(), q.stride(0), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
+        _dev(table, "table", torch.int32), table.shape[1],
+        _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
+        _dev(slots, "slots", torch.int32), T, nh, nkv, d, page_size, num_pages, float(scale),
+        int(window), _code(out, "out"), _stream()), "kvc_paged_attention")
+
+
+def gemm_f32(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None) -> None:
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape != (N, K) or out.shape != (M, N) or a.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm_f32: shapes do not match")
+    for t, name in ((a, "a"), (out, "out")):
+        if t.dtype != torch.float32 or not t.is_cuda:
+            raise KernelError(f"gemm_f32: {name} must be a float32 GPU tensor")
+    _check(load().kvc_gemm_f32(out.data_ptr(), a.data_ptr(), _dev(w, "w", torch.float32),
+                               None if bias is None else _dev(bias, "bias", torch.float32),
+                               M, N, K, a.stride(0), out.stride(0), _stream()), "kvc_gemm_f32")
+
+
+def linear(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -> None:
+    """``out = x @ w.T (+ bias)``.  float32 runs the library's own true-float32 kernel;
+    bfloat16 runs the vendor matrix product through torch (float32 accumulation)."""
+    if x.dtype == torch.float32:
+        gemm_f32(out, x, w, bias)
+        return
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not x.is_cuda:
+        raise KernelError(f"linear: unsupported operands {x.dtype}/{w.dtype} on {x.device}")
+    if x.shape[0] == 0:
+        return
+    if bias is None:
+        torch.mm(x, w.t(), out=out)
+    else:
+        torch.addmm(bias, x, w.t(), out=out)
+
+
+def table_update(table: torch.Tensor, triples: torch.Tensor, n: int) -> None:
+    if triples.numel() < 3 * n:
+        raise KernelError("table_update: triples too short")
+    _check(load().kvc_table_update(_dev(table, "table", torch.int32), table.shape[1], table.shape[0],
+                                   _dev(triples, "triples", torch.int32), n, _stream()),
+           "kvc_table_update")
+
+
+def argmax(out: torch.Tensor, logits: torch.Tensor) -> None:
+    S, V = logits.shape
+    if out.numel() < S or logits.stride(1) != 1 or logits.dtype != torch.float32 or not logits.is_cuda:
+        raise KernelError("argmax: expects float32 GPU logits [S, V] and S outputs")
+    _check(load().kvc_argmax(_dev(out, "out", torch.int32), logits.data_ptr(), S, V,
+                             logits.stride(0), _stream()), "kvc_argmax")
+
+
+def sample(out: torch.Tensor, logits: torch.Tensor, *, temperature: torch.Tensor,
+           top_k: torch.Tensor, top_p: torch.Tensor, seed_lo: torch.Tensor, seed_hi: torch.Tensor,
+           index: torch.Tensor) -> None:
+    S, V = logits.shape
+    if logits.stride(1) != 1 or logits.dtype != torch.float32 or not logits.is_cuda:
+        raise KernelError("sample: expects float32 GPU logits [S, V]")
+    for t, name in ((out, "out"), (temperature, "temperature"), (top_k, "top_k"), (top_p, "top_p"),
+                    (seed_lo, "seed_lo"), (seed_hi, "seed_hi"), (index, "index")):
+        if t.numel() < S or t.element_size() != 4:
+            raise KernelError(f"sample: {name} must hold {S} 32-bit values")
+    _check(load().kvc_sample(_dev(out, "out", torch.int32), logits.data_ptr(), S, V, logits.stride(0),
+                             _dev(temperature, "temperature", torch.float32),
+                             _dev(top_k, "top_k", torch.int32), _dev(top_p, "top_p", torch.float32),
+                             _dev(seed_lo, "seed_lo"), _dev(seed_hi, "seed_hi"), _dev(index, "index"),
+                             _stream()), "kvc_sample")

@@ -1,0 +1,90 @@
+"""Grouped-query attention over the paged cache.
+
+Reference: kvcore/model/models/llama3.py:48-104 (stacked qkv projection with rows in
+the order q, k, v; rotation of q and k; attention; output projection) and
+kvcore/model/attn_backend/torch_paged.py:70-117 (keys and values are written to their
+page slots first, then every query reads keys ``0..position`` back from the cache).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from kvcore_amd.ops import library as ops
+
+from .base import CacheNeed, Mixer, ParamSource, ParamSpec, PositionEncoding, register_mixer
+
+
+class PagedAttention(Mixer):
+    """``scale`` is a parameter (the reference fixes ``head_dim ** -0.5`` at
+    llama3.py:60); ``window`` 0 attends to every earlier token."""
+
+    def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 scale: float, bias: bool = False, window: int = 0,
+                 position: PositionEncoding | None = None) -> None:
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if head_dim % 16 or head_dim > 256:
+            raise ValueError(f"head size {head_dim} is not supported (multiples of 16 up to 256)")
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.scale = scale
+        self.bias = bias
+        self.window = window
+        self.position = position
+        self.q_size = num_heads * head_dim
+        self.kv_size = num_kv_heads * head_dim
+
+    def param_specs(self) -> list[ParamSpec]:
+        total = self.q_size + 2 * self.kv_size
+
+        def stacked(suffix: str) -> tuple[ParamSource, ...]:
+            return (
+                ParamSource(f"q_proj.{suffix}", 0, self.q_size),
+                ParamSource(f"k_proj.{suffix}", self.q_size, self.kv_size),
+                ParamSource(f"v_proj.{suffix}", self.q_size + self.kv_size, self.kv_size),
+            )
+
+        specs = [
+            ParamSpec("qkv_proj.weight", (total, self.hidden_size), sources=stacked("weight")),
+            ParamSpec("o_proj.weight", (self.hidden_size, self.q_size)),
+        ]
+        if self.bias:
+            specs.append(ParamSpec("qkv_proj.bias", (total,), init="zeros", sources=stacked("bias")))
+            specs.append(ParamSpec("o_proj.bias", (self.hidden_size,), init="zeros"))
+        return specs
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def forward(self, x: torch.Tensor, ctx, call) -> torch.Tensor:
+        p = self.params
+        qkv = ctx.buf("attn_qkv", self.q_size + 2 * self.kv_size)
+        ops.linear(qkv, x, p["qkv_proj.weight"], p.get("qkv_proj.bias"))
+
+        group = ctx.groups[call.group_index]
+        k_cache, v_cache = group.planes(call.cache_index)
+        rot = self.position.rotary(ctx) if self.position is not None else None
+        if rot is None:
+            cos = sin = ctx.buffers.get("rope_none", ctx.num_tokens, 0, torch.float32)
+            rot_dim, interleaved = 0, False
+        else:
+            cos, sin, rot_dim, interleaved = rot.cos, rot.sin, rot.rot_dim, rot.interleaved
+        ops.rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim, interleaved=interleaved,
+                          positions=ctx.positions, token_req=ctx.token_req, slots=ctx.slots,
+                          table=group.table, nh=self.num_heads, nkv=self.num_kv_heads,
+                          d=self.head_dim, write_kv=call.write_cache)
+
+        attn = ctx.buf("attn_out", self.q_size)
+        ops.paged_attention(attn, qkv, k_cache, v_cache, table=group.table, positions=ctx.positions,
+                            token_req=ctx.token_req, slots=ctx.slots, nh=self.num_heads,
+                            nkv=self.num_kv_heads, d=self.head_dim, scale=self.scale,
+                            window=self.window)
+        out = ctx.buf("mixer_out", self.hidden_size)
+        ops.linear(out, attn, p["o_proj.weight"], p.get("o_proj.bias"))
+        return out
+
+
+register_mixer("paged_attention", PagedAttention)

@@ -1,0 +1,230 @@
+"""Interfaces of the parts a model is put together from, and their registries.
+
+A model is data: a ``ModelSpec`` lists layers, each layer names its parts by kind with
+their sizes and constants as plain arguments, and a schedule lists the order in which
+layers run.  The kinds are looked up here, so a new mixer, feed-forward, norm,
+position encoding or block arrangement is one class and one ``register_*`` call; no
+part knows which model it is in.
+
+The reference composes fixed classes instead (kvcore/model/models/llama3.py:107-142);
+its parts take their constants partly as parameters (layer/attention.py:19-31,
+layer/rmsnorm.py:8) and partly from the config object (layer/rotary_embedding.py:53).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import TYPE_CHECKING, Any, Callable
+
+import torch
+
+if TYPE_CHECKING:
+    from kvcore_amd.engine.context import LayerCall, StepContext
+
+
+# ------------------------------------------------------------------------ parameters
+@dataclass(frozen=True)
+class ParamSource:
+    """One checkpoint tensor that fills rows ``[row, row + rows)`` of a parameter.
+    ``name`` is relative to the part's checkpoint prefix."""
+
+    name: str
+    row: int
+    rows: int
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """A parameter a part owns.
+
+    ``kind``: ``"matrix"`` is kept in the model dtype; ``"vector"`` is always float32
+    (norm gains and the like, whatever the file stores); ``"table"`` is int32.
+    ``init`` names the rule of the random-weights mode: ``"normal"`` N(0, 0.02),
+    ``"gain"`` 1 + N(0, 0.1), ``"zeros"``.
+    ``sources`` empty means one checkpoint tensor of the same name and shape.
+    ``alias_of`` names another parameter (by full name) whose storage this one shares;
+    a checkpoint tensor for an alias is optional.
+    """
+
+    name: str
+    shape: tuple[int, ...]
+    kind: str = "matrix"
+    init: str = "normal"
+    sources: tuple[ParamSource, ...] = ()
+
+    def resolved_sources(self) -> tuple[ParamSource, ...]:
+        return self.sources or (ParamSource(self.name, 0, self.shape[0]),)
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """Paged memory that grows with the sequence: keys and values of ``num_kv_heads``
+    heads of ``head_dim``.  ``window`` 0 keeps every token, ``w > 0`` only the last
+    ``w`` (pages wholly behind the window are given back during the request)."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size, kept in a slot array ``[max_seqs, *shape]``."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass(frozen=True)
+class Runtime:
+    """What a part needs to know about where it runs."""
+
+    dtype: torch.dtype
+    device: torch.device
+
+
+class Part:
+    """Base of all parts: declares parameters, receives them bound to device tensors."""
+
+    def param_specs(self) -> list[ParamSpec]:
+        return []
+
+    def setup(self, runtime: Runtime) -> None:
+        """Called once after construction, before parameters are bound."""
+        self.runtime = runtime
+
+    def bind(self, params: dict[str, torch.Tensor]) -> None:
+        """``params`` maps the local names of ``param_specs`` to device tensors."""
+        self.params = params
+
+
+class Norm(Part):
+    """``forward_fused`` adds ``delta`` (may be None) into the float32 ``residual`` in
+    place and writes the normalised rows into ``out`` (model dtype)."""
+
+    def forward_fused(self, out: torch.Tensor, residual: torch.Tensor,
+                      delta: torch.Tensor | None) -> None:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Position information.  ``prepare`` runs once per step before any layer.
+    ``rotary`` returns what a mixer needs to rotate queries and keys, or None if this
+    encoding does not rotate; ``embed`` may change the embedded rows in place."""
+
+    def prepare(self, ctx: "StepContext") -> None:
+        pass
+
+    def rotary(self, ctx: "StepContext") -> "RotaryTables | None":
+        return None
+
+    def embed(self, residual: torch.Tensor, ctx: "StepContext") -> None:
+        pass
+
+
+@dataclass
+class RotaryTables:
+    cos: torch.Tensor  # [>= T, rot_dim / 2] float32
+    sin: torch.Tensor
+    rot_dim: int
+    interleaved: bool
+
+
+class Mixer(Part):
+    """Mixes information across the tokens of a request.  ``x`` is ``[T, hidden]`` in
+    the model dtype; the result has the same shape and may live in a step buffer."""
+
+    def cache_need(self) -> CacheNeed | None:
+        return None
+
+    def state_need(self) -> StateNeed | None:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: "StepContext", call: "LayerCall") -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx: "StepContext", call: "LayerCall") -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of norms, mixer and feed-forward around the residual stream.
+    ``forward`` takes the pending ``delta`` (output of the previous block not yet added,
+    or None) and the float32 ``residual``, and returns the new pending delta."""
+
+    def __init__(self, *, mixer: Mixer, ffn: FeedForward, norms: dict[str, Norm]) -> None:
+        self.mixer = mixer
+        self.ffn = ffn
+        self.norms = norms
+
+    def children(self) -> dict[str, Part]:
+        """Checkpoint sub-prefix -> part."""
+        raise NotImplementedError
+
+    def forward(self, delta: torch.Tensor | None, residual: torch.Tensor, ctx: "StepContext",
+                call: "LayerCall") -> torch.Tensor:
+        raise NotImplementedError
+
+
+# -------------------------------------------------------------------------- registry
+@dataclass(frozen=True)
+class PartSpec:
+    """A part chosen by kind, with its sizes and constants."""
+
+    kind: str
+    args: dict[str, Any] = field(default_factory=dict)
+
+
+class _Registry:
+    def __init__(self, what: str) -> None:
+        self.what = what
+        self._items: dict[str, Callable[..., Any]] = {}
+
+    def register(self, kind: str, factory: Callable[..., Any], *, replace: bool = False) -> None:
+        if kind in self._items and not replace:
+            raise ValueError(f"{self.what} kind {kind!r} is already registered")
+        self._items[kind] = factory
+
+    def build(self, spec: PartSpec, **extra: Any) -> Any:
+        try:
+            factory = self._items[spec.kind]
+        except KeyError:
+            raise ValueError(
+                f"Unknown {self.what} kind {spec.kind!r}. Registered: {sorted(self._items)}"
+            ) from None
+        return factory(**spec.args, **extra)
+
+    def kinds(self) -> list[str]:
+        return sorted(self._items)
+
+    def unregister(self, kind: str) -> None:
+        self._items.pop(kind, None)
+
+
+MIXERS = _Registry("mixer")
+FEED_FORWARDS = _Registry("feed-forward")
+NORMS = _Registry("norm")
+POSITION_ENCODINGS = _Registry("position encoding")
+BLOCKS = _Registry("block")
+
+
+def register_mixer(kind: str, factory: Callable[..., Mixer], **kw: Any) -> None:
+    MIXERS.register(kind, factory, **kw)
+
+
+def register_feed_forward(kind: str, factory: Callable[..., FeedForward], **kw: Any) -> None:
+    FEED_FORWARDS.register(kind, factory, **kw)
+
+
+def register_norm(kind: str, factory: Callable[..., Norm], **kw: Any) -> None:
+    NORMS.register(kind, factory, **kw)
+
+
+def register_position_encoding(kind: str, factory: Callable[..., PositionEncoding], **kw: Any) -> None:
+    POSITION_ENCODINGS.register(kind, factory, **kw)
+
+
+def register_block(kind: str, factory: Callable[..., Block], **kw: Any) -> None:
+    BLOCKS.register(kind, factory, **kw)

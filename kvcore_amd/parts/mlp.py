@@ -1,0 +1,48 @@
+"""Gated feed-forward: ``down(silu(gate(x)) * up(x))`` with gate and up stacked.
+
+Reference: kvcore/model/models/llama3.py:25-45 (gate rows first, then up rows) and
+kvcore/model/layer/activation.py:14-16.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from kvcore_amd.ops import library as ops
+
+from .base import FeedForward, ParamSource, ParamSpec, register_feed_forward
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, *, hidden_size: int, intermediate_size: int, bias: bool = False) -> None:
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.bias = bias
+
+    def param_specs(self) -> list[ParamSpec]:
+        I, H = self.intermediate_size, self.hidden_size
+
+        def stacked(suffix: str) -> tuple[ParamSource, ...]:
+            return (ParamSource(f"gate_proj.{suffix}", 0, I), ParamSource(f"up_proj.{suffix}", I, I))
+
+        specs = [
+            ParamSpec("gate_up_proj.weight", (2 * I, H), sources=stacked("weight")),
+            ParamSpec("down_proj.weight", (H, I)),
+        ]
+        if self.bias:
+            specs.append(ParamSpec("gate_up_proj.bias", (2 * I,), init="zeros", sources=stacked("bias")))
+            specs.append(ParamSpec("down_proj.bias", (H,), init="zeros"))
+        return specs
+
+    def forward(self, x: torch.Tensor, ctx, call) -> torch.Tensor:
+        p = self.params
+        gate_up = ctx.buf("ffn_gate_up", 2 * self.intermediate_size)
+        ops.linear(gate_up, x, p["gate_up_proj.weight"], p.get("gate_up_proj.bias"))
+        act = ctx.buf("ffn_act", self.intermediate_size)
+        ops.silu_mul(act, gate_up)
+        out = ctx.buf("ffn_out", self.hidden_size)
+        ops.linear(out, act, p["down_proj.weight"], p.get("down_proj.bias"))
+        return out
+
+
+register_feed_forward("swiglu", SwiGLU)
