@@ -23,3 +23,11 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    from tests import helpers
+
+    for label, (ratio, abs_err) in sorted(helpers.ERROR_STATS.items()):
+        terminalreporter.write_line(
+            f"[numerics] {label}: worst error {abs_err:.3e}, {ratio:.2f} of its bound")

@@ -77,5 +77,16 @@ def tolerance(dtype: torch.dtype) -> dict:
     relative per operation over a few hundred operations.  bfloat16: activations are
     rounded to 8 bits of mantissa (2^-9 relative) at about ten places per layer."""
     if dtype == torch.float32:
-        return dict(atol=2e-5, rtol=1e-4)
+        return dict(atol=5e-6, rtol=2e-5)
     return dict(atol=8e-3, rtol=2e-2)
+
+
+ERROR_STATS: dict[str, list[float]] = {}
+
+
+def note_error(label: str, ratio: float, abs_err: float) -> None:
+    """Keeps the worst error seen per label (largest fraction of its bound, largest
+    absolute value); the terminal summary prints them."""
+    cur = ERROR_STATS.setdefault(label, [0.0, 0.0])
+    cur[0] = max(cur[0], ratio)
+    cur[1] = max(cur[1], abs_err)

@@ -68,11 +68,13 @@ def collect(session, steps):
 def compare(got, expect_by_id, dtype):
     tol = tolerance(dtype)
     assert got, "nothing was compared"
+    from tests import helpers
     for (rid, pos), row in sorted(got.items()):
         ref = expect_by_id[rid][pos]
         assert torch.isfinite(row).all(), f"non-finite logits at {rid}:{pos}"
         err = (row - ref).abs()
         bound = tol["atol"] + tol["rtol"] * ref.abs()
+        helpers.note_error(str(dtype), float((err / bound).max()), float(err.max()))
         if not (err <= bound).all():
             worst = int(torch.argmax(err - bound))
             raise AssertionError(
@@ -180,7 +182,8 @@ def mixed_trace(token_lists, seed):
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_mixed_batches_with_page_reuse(models, name, dtype):
     folder, cfg, weights, page = models[name]
-    lens = PROMPT_LENS[name] + [PROMPT_LENS[name][1] + 3, PROMPT_LENS[name][2] + 1]
+    base = PROMPT_LENS[name]
+    lens = base + [n + 3 for n in base] + [base[-1] + 17, base[0] + 1]
     token_lists = {f"q{i}": random_tokens(n + EXTRA, cfg["vocab_size"], seed=400 + i) for i, n in enumerate(lens)}
     rounded = sorted((-(-len(t) // 64) * 64 for t in token_lists.values()), reverse=True)
     max_tokens = sum(rounded[:4])  # the four largest live at once; the rest must reuse pages
