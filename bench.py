@@ -1,0 +1,199 @@
+"""Decode and prefill throughput of the Llama-3-8B shape with random weights on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode step of the whole engine (scheduler, step function, sampler) at
+batch 8 from 512-token prompts, context limit 8192.  One JSON line is printed:
+``value`` is decoded tokens a second; ``prefill`` is a 2,048-token prompt in one step;
+``roofline`` prices the decode step's mandatory reads (every weight once, the live
+requests' cache) against 8 TB/s; ``points`` holds decode at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import random
+import sys
+import time
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+LLAMA3_8B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 32, "hidden_size": 4096, "num_attention_heads": 32,
+    "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 14336, "vocab_size": 128256,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
+    "tie_word_embeddings": False, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192,
+    "hidden_act": "silu",
+}
+CONTEXT_LEN = 8192
+PROMPT_LEN = 512
+NEW_TOKENS = 256
+PREFILL_TOKENS = 2048
+PAGE_SIZE = 16
+HBM_PEAK = 8.0e12          # bytes/s, MI355X
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=128)
+    p.add_argument("--warmup", type=int, default=16)
+    p.add_argument("--batch", type=int, default=8)
+    p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
+    p.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    p.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    return p.parse_args()
+
+
+def weight_bytes_per_step(cfg, esize):
+    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    nh, nkv, d, L = (cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"],
+                     cfg["num_hidden_layers"])
+    per_layer = (nh + 2 * nkv) * d * H + nh * d * H + 3 * I * H
+    return (L * per_layer + V * H) * esize
+
+
+def kv_bytes(cfg, batch, ctx, esize):
+    return batch * ctx * 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"] * cfg["head_dim"] * esize
+
+
+def prefill_flops(cfg, T, S=1):
+    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    nh, nkv, d, L = (cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"],
+                     cfg["num_hidden_layers"])
+    per_layer = (nh + 2 * nkv) * d * H + nh * d * H + 3 * I * H
+    return 2 * T * L * per_layer + 4 * d * nh * L * T * (T + 1) // 2 + 2 * S * V * H
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    import torch
+
+    from kvcore_amd import (CacheConfig, DeviceConfig, KVCoreConfig, LoadConfig, ModelConfig,
+                            SamplingParams, SchedulerConfig)
+    from kvcore_amd.engine.engine_core import EngineCore
+    from kvcore_amd.engine.runner import build_model
+
+    cfg = dict(LLAMA3_8B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers is not None:
+        cfg["num_hidden_layers"] = args.layers
+    dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
+    esize = 2 if args.dtype == "bf16" else 4
+    device = "cuda:0"
+    torch.cuda.set_device(0)
+
+    t0 = time.perf_counter()
+    model = build_model(".", dtype, device, load_format="random", seed=0, config_override=cfg)
+    print(f"[bench] model built in {time.perf_counter() - t0:.1f} s, "
+          f"{model.num_param_bytes() / 2**30:.2f} GiB", file=sys.stderr, flush=True)
+
+    max_seqs = 64
+    pages_per_seq = -(-(PREFILL_TOKENS + NEW_TOKENS + PROMPT_LEN) // PAGE_SIZE)
+    engine = EngineCore(KVCoreConfig(
+        model_config=ModelConfig(model=".", dtype=args.dtype, max_model_len=CONTEXT_LEN),
+        load_config=LoadConfig(load_format="random", seed=0),
+        cache_config=CacheConfig(block_size=PAGE_SIZE, num_gpu_blocks=max_seqs * pages_per_seq + 1),
+        scheduler_config=SchedulerConfig(max_num_seqs=max_seqs, max_num_scheduled_tokens=PREFILL_TOKENS,
+                                         max_num_partial_prefills=max_seqs,
+                                         max_long_partial_prefills=max_seqs),
+        device_config=DeviceConfig(device=device),
+    ), model=model)
+    rng = random.Random(0)
+    vocab = cfg["vocab_size"]
+    counter = [0]
+
+    def new_request(n_prompt, n_new):
+        counter[0] += 1
+        rid = f"bench-{counter[0]}"
+        ids = [rng.randrange(vocab) for _ in range(n_prompt)]
+        engine.add_request(rid, SamplingParams(max_tokens=n_new, temperature=0.0, ignore_eos=True),
+                           prompt_token_ids=ids)
+        return rid
+
+    def drain():
+        while engine.has_unfinished_requests():
+            engine.step()
+
+    def decode_run(batch, steps, warmup):
+        """tokens/s over exactly `steps` decode steps at `batch`, after `warmup` of them."""
+        slack = -(-batch * PROMPT_LEN // PREFILL_TOKENS) + 2  # steps others decode while prompts run
+        for _ in range(batch):
+            new_request(PROMPT_LEN, warmup + steps + 1 + slack)
+        # prompts first; a request samples its first token when its prompt ends
+        while any(r.num_computed_tokens < r.num_prompt_tokens
+                  for r in engine.scheduler.requests.values()):
+            engine.step()
+        for _ in range(warmup):
+            engine.step()
+        ctx_start = PROMPT_LEN + 1 + warmup
+        torch.cuda.synchronize()
+        t_start = time.perf_counter()
+        for _ in range(steps):
+            engine.step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t_start
+        engine.abort_requests(None)
+        mean_ctx = ctx_start + steps / 2
+        return batch * steps / elapsed, elapsed / steps, mean_ctx
+
+    def prefill_run():
+        times = []
+        for i in range(4):
+            new_request(PREFILL_TOKENS, 1)
+            torch.cuda.synchronize()
+            t_start = time.perf_counter()
+            engine.step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t_start)
+            drain()
+        return sorted(times[1:])[1]  # median of the three after the warm-up run
+
+    value, sec_per_step, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
+    bytes_step = weight_bytes_per_step(cfg, esize) + kv_bytes(cfg, args.batch, mean_ctx, esize)
+    achieved = bytes_step / sec_per_step
+    result = {
+        "metric": "decode tok/s (Llama-3-8B shape, batch 8, 512-token prompts)",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {
+            "model": "llama-3-8b-shape-random", "layers": cfg["num_hidden_layers"],
+            "layers_full": full_layers, "hidden": cfg["hidden_size"],
+            "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+            "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"],
+            "vocab": cfg["vocab_size"], "global_batch": args.batch, "seq_len": CONTEXT_LEN,
+            "prompt_len": PROMPT_LEN, "new_tokens": NEW_TOKENS, "page_size": PAGE_SIZE,
+            "prefill_tokens": PREFILL_TOKENS, "parallelism": "single-gpu",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)},
+    }
+    if not args.no_points:
+        sec = prefill_run()
+        flops = prefill_flops(cfg, PREFILL_TOKENS)
+        result["prefill"] = {"value": round(PREFILL_TOKENS / sec, 1), "tokens": PREFILL_TOKENS,
+                             "ms": round(sec * 1e3, 3),
+                             "frac": round(flops / sec / PEAK_FLOPS[args.dtype], 4)}
+        points = {}
+        for b in (1, 64):
+            steps = max(16, min(args.steps, 64))
+            v, _, _ = decode_run(b, steps, min(args.warmup, 8))
+            points[f"decode_b{b}"] = round(v, 2)
+        result["points"] = points
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,93 @@
+"""Turns float32 logits into token ids on the GPU.
+
+Reference: kvcore/sample/sampler.py:86-167: float logits; rows whose temperature is
+below 1e-5 take the argmax; the others are divided by their temperature, filtered by
+top-k and top-p, and drawn as ``argmax(softmax / q)`` with ``q ~ Exp(1)``.  The
+reference seeds a fresh generator inside every call (:53-57,185-188), so a seeded
+request would draw the same noise for every token; here the noise of a request's
+``index``-th output token is a function of (seed, index) alone, so a seeded run is
+reproducible, independent of what else is in the batch, and fresh at every token.
+"""
+
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from kvcore_amd.ops import library as ops
+
+from .params import SamplingParams
+
+GREEDY_EPS = 1e-5  # sampler.py:11
+
+
+@dataclass(frozen=True)
+class SamplingRow:
+    """One logits row's options: ``seed`` is the request's 64-bit seed (already
+    resolved), ``index`` the number of tokens the request has produced so far."""
+
+    params: SamplingParams
+    seed: int
+    index: int
+
+
+class Sampler:
+    def __init__(self, device: torch.device | str, max_rows: int, engine_seed: int | None = None) -> None:
+        self.device = torch.device(device)
+        self.max_rows = max_rows
+        self.engine_seed = int.from_bytes(os.urandom(8), "little") if engine_seed is None else engine_seed
+        self._requests_seen = 0
+        n = max_rows
+        self._host = torch.empty(6 * n, dtype=torch.int32, pin_memory=True)
+        self._host_np = self._host.numpy()
+        self._dev = torch.empty(6 * n, dtype=torch.int32, device=self.device)
+        self._out_dev = torch.empty(n, dtype=torch.int32, device=self.device)
+        self._out_host = torch.empty(n, dtype=torch.int32, pin_memory=True)
+
+    def resolve_seed(self, params: SamplingParams) -> int:
+        """The request's own seed, or one derived from the engine's seed and the order of
+        arrival (the reference draws unseeded rows from torch's global generator)."""
+        self._requests_seen += 1
+        if params.seed is not None:
+            return params.seed & 0xFFFFFFFFFFFFFFFF
+        x = (self.engine_seed + 0x9E3779B97F4A7C15 * self._requests_seen) & 0xFFFFFFFFFFFFFFFF
+        x ^= x >> 31
+        return (x * 0xBF58476D1CE4E5B9) & 0xFFFFFFFFFFFFFFFF
+
+    def sample(self, logits: torch.Tensor, rows: Sequence[SamplingRow]) -> list[int]:
+        S = len(rows)
+        if logits.shape[0] != S:
+            raise ValueError(f"{S} sampling rows for {logits.shape[0]} logits rows")
+        if S == 0:
+            return []
+        if S > self.max_rows:
+            raise ValueError(f"{S} rows exceed the sampler's capacity {self.max_rows}")
+        out = self._out_dev[:S]
+        if all(r.params.temperature < GREEDY_EPS for r in rows):
+            ops.argmax(out, logits)
+        else:
+            n = self.max_rows
+            buf = self._host_np
+            fview = buf.view(np.float32)
+            uview = buf.view(np.uint32)
+            V = logits.shape[1]
+            for i, r in enumerate(rows):
+                p = r.params
+                fview[i] = p.temperature
+                buf[n + i] = 0 if p.top_k is None else min(p.top_k, V)
+                fview[2 * n + i] = p.top_p
+                uview[3 * n + i] = r.seed & 0xFFFFFFFF
+                uview[4 * n + i] = (r.seed >> 32) & 0xFFFFFFFF
+                uview[5 * n + i] = r.index & 0xFFFFFFFF
+            self._dev.copy_(self._host, non_blocking=True)
+            d = self._dev
+            ops.sample(out, logits, temperature=d[:n].view(torch.float32), top_k=d[n:2 * n],
+                       top_p=d[2 * n:3 * n].view(torch.float32), seed_lo=d[3 * n:4 * n],
+                       seed_hi=d[4 * n:5 * n], index=d[5 * n:6 * n])
+        self._out_host[:S].copy_(out, non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        return self._out_host[:S].tolist()
