@@ -1,0 +1,110 @@
+from __future__ import annotations
+
+import json
+
+import pytest
+
+from kvcore_amd.config.engine_config import (CacheConfig, KVCoreConfig, ModelConfig, SchedulerConfig,
+                                             canonical_dtype)
+from kvcore_amd.config.model_config import ConfigError, LlamaConfig, RopeScaling, read_config_json
+from kvcore_amd.models.llama import llama_spec
+from kvcore_amd.registry import (MODEL_REGISTRY, register_architecture, resolve_architecture,
+                                 unregister_architecture)
+from tests.helpers import TINY_A, TINY_B, TINY_C
+
+
+def test_every_size_comes_from_the_file():
+    for raw in (TINY_A, TINY_B, TINY_C):
+        c = LlamaConfig.from_dict(raw)
+        assert c.vocab_size == raw["vocab_size"] and c.hidden_size == raw["hidden_size"]
+        assert c.num_hidden_layers == raw["num_hidden_layers"]
+        assert c.num_key_value_heads == raw["num_key_value_heads"] and c.head_dim == raw["head_dim"]
+        assert c.rms_norm_eps == raw["rms_norm_eps"] and c.rope_theta == raw["rope_theta"]
+        spec = llama_spec(c)
+        attn = spec.layers[0].mixer.args
+        assert attn["scale"] == raw["head_dim"] ** -0.5  # llama3.py:60
+        assert spec.layers[0].norms["input_layernorm"].args["eps"] == raw["rms_norm_eps"]
+        assert spec.layers[0].ffn.args["intermediate_size"] == raw["intermediate_size"]
+        assert spec.tie_word_embeddings == raw["tie_word_embeddings"]
+        assert len(spec.layers) == raw["num_hidden_layers"]
+        assert LlamaConfig.from_dict(c.to_dict()) == c
+
+
+def test_defaults_follow_the_reference():
+    raw = {k: v for k, v in TINY_A.items() if k not in ("num_key_value_heads", "head_dim", "rope_theta")}
+    c = LlamaConfig.from_dict(raw)
+    assert c.num_key_value_heads == c.num_attention_heads  # engine_core.py:164
+    assert c.head_dim == c.hidden_size // c.num_attention_heads  # llama3.py:59
+    assert c.rope_theta == 10000.0  # rotary_embedding.py:49
+    raw["rope_parameters"] = {"rope_theta": 123.0}
+    assert LlamaConfig.from_dict(raw).rope_theta == 123.0  # rotary_embedding.py:40-43
+
+
+@pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers",
+                                 "num_attention_heads", "rms_norm_eps", "max_position_embeddings"])
+def test_a_missing_required_key_is_named(key):
+    raw = {k: v for k, v in TINY_A.items() if k != key}
+    with pytest.raises(ConfigError, match=key):
+        LlamaConfig.from_dict(raw)
+
+
+def test_refused_values():
+    with pytest.raises(ConfigError, match="activation"):
+        LlamaConfig.from_dict({**TINY_A, "hidden_act": "gelu"})  # llama3.py:28-31
+    with pytest.raises(ConfigError, match="rope_type"):
+        LlamaConfig.from_dict({**TINY_A, "rope_scaling": {"rope_type": "yarn", "factor": 2.0}})
+    with pytest.raises(ConfigError, match="multiple"):
+        LlamaConfig.from_dict({**TINY_A, "num_key_value_heads": 3})
+    with pytest.raises(ConfigError, match="low_freq_factor"):
+        LlamaConfig.from_dict({**TINY_A, "rope_scaling": {"rope_type": "llama3", "factor": 2.0}})
+    assert RopeScaling.from_dict({"rope_type": "default"}) == RopeScaling()
+
+
+def test_eos_may_be_an_int_or_a_list():
+    assert LlamaConfig.from_dict({**TINY_A, "eos_token_id": 7}).eos_token_ids == (7,)
+    assert LlamaConfig.from_dict({**TINY_A, "eos_token_id": [7, 9]}).eos_token_ids == (7, 9)
+
+
+def test_registry_key_is_the_architecture_name_with_model_type_as_fallback():
+    assert resolve_architecture(TINY_A).name == "LlamaForCausalLM"
+    assert resolve_architecture({"model_type": "llama"}).name == "LlamaForCausalLM"
+    with pytest.raises(ValueError, match="Supported"):
+        resolve_architecture({"architectures": ["NoSuchModel"], "model_type": "none"})
+    with pytest.raises(ValueError, match="already registered"):
+        register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, llama_spec)
+    register_architecture("ToyForTest", LlamaConfig.from_dict, llama_spec)
+    try:
+        assert resolve_architecture({"architectures": ["ToyForTest"]}).name == "ToyForTest"
+    finally:
+        unregister_architecture("ToyForTest")
+    assert "ToyForTest" not in MODEL_REGISTRY
+
+
+def test_read_config_json(tmp_path):
+    with pytest.raises(FileNotFoundError):
+        read_config_json(tmp_path / "missing")
+    with pytest.raises(FileNotFoundError):
+        read_config_json(tmp_path)
+    (tmp_path / "config.json").write_text(json.dumps(TINY_A))
+    assert read_config_json(tmp_path)["vocab_size"] == 256
+
+
+def test_engine_config_validation():
+    """kvcore/config.py:15-93."""
+    assert canonical_dtype("torch.bfloat16") == "bfloat16" and canonical_dtype("fp32") == "float32"
+    with pytest.raises(ValueError):
+        canonical_dtype("float16")
+    with pytest.raises(ValueError):
+        ModelConfig(model="x", max_model_len=0)
+    with pytest.raises(ValueError):
+        CacheConfig(block_size=0)
+    with pytest.raises(ValueError):
+        CacheConfig(gpu_memory_utilization=0.0)
+    with pytest.raises(ValueError):
+        SchedulerConfig(max_num_seqs=0)
+    with pytest.raises(ValueError):
+        SchedulerConfig(long_prefill_token_threshold=-1)
+    cfg = KVCoreConfig(ModelConfig(model="x", dtype="bf16"))
+    assert cfg.model_config.dtype == "bfloat16"
+    assert (cfg.cache_config.block_size, cfg.scheduler_config.max_num_seqs,
+            cfg.scheduler_config.max_num_scheduled_tokens) == (16, 8, 512)
