@@ -1,0 +1,417 @@
+"""Each kernel alone against a plain float64/float32 torch computation of the same op,
+at sizes other than the engine's (widths that are no power of two, odd row counts)."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+from tests.plain import llama as plain
+from tests.plain import sampling as plain_sampling
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from kvcore_amd.ops import library
+
+    library.load()
+    return library
+
+
+def tol(dtype):
+    return dict(atol=2e-6, rtol=2e-6) if dtype == torch.float32 else dict(atol=1e-2, rtol=1e-2)
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(ops, dtype):
+    V, H = 37, 100
+    table = rnd(V, H, dtype=dtype)
+    ids = torch.tensor([0, 36, 5, 5, 40, -1], dtype=torch.int32, device=DEV)
+    out = torch.zeros(6, H, device=DEV)
+    ops.embed(out, table, ids)
+    assert torch.equal(out[:4], table.float()[ids[:4].long()])
+    assert torch.isnan(out[4:]).all()  # an id outside the table is loud, not a stray read
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H", [96, 200, 4100])
+def test_add_rmsnorm(ops, dtype, H):
+    T, eps = 5, 1e-5
+    residual = rnd(T, H, seed=1)
+    delta = rnd(T, H, dtype=dtype, seed=2)
+    w = 1 + 0.1 * rnd(H, seed=3)
+    want_res = residual.double() + delta.double()
+    want = plain.rms_norm(want_res, w.double(), eps)
+    out = torch.empty(T, H, dtype=dtype, device=DEV)
+    res = residual.clone()
+    ops.add_rmsnorm(out, res, delta, w, eps)
+    assert torch.allclose(res.double(), want_res, atol=1e-6)  # the sum stays float32
+    assert torch.allclose(out.double(), want, **tol(dtype))
+    res2 = residual.clone()
+    ops.add_rmsnorm(out, res2, None, w, eps)
+    assert torch.equal(res2, residual)
+    assert torch.allclose(out.double(), plain.rms_norm(residual.double(), w.double(), eps), **tol(dtype))
+    ops.residual_add(res2, delta)
+    assert torch.allclose(res2.double(), want_res, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_on_strided_rows(ops, dtype):
+    big = rnd(7, 300, dtype=dtype)
+    x = big[:, 20:116]
+    w = 1 + 0.1 * rnd(96, seed=4)
+    out = torch.empty(7, 96, dtype=dtype, device=DEV)
+    ops.rmsnorm(out, x, w, 1e-6)
+    assert torch.allclose(out.double(), plain.rms_norm(x.double(), w.double(), 1e-6), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(ops, dtype):
+    gu = rnd(9, 2 * 177, dtype=dtype, scale=3.0)
+    out = torch.empty(9, 177, dtype=dtype, device=DEV)
+    ops.silu_mul(out, gu)
+    assert torch.allclose(out.double(), plain.silu_and_mul(gu.double()), **tol(dtype))
+
+
+def test_gather_rows_and_to_float(ops):
+    src = rnd(10, 50)
+    rows = torch.tensor([9, 0, 3, 3], dtype=torch.int32, device=DEV)
+    out = torch.empty(4, 50, dtype=torch.bfloat16, device=DEV)
+    ops.gather_rows(out, src, rows)
+    assert torch.equal(out, src[rows.long()].to(torch.bfloat16))
+    back = torch.empty(4, 50, device=DEV)
+    ops.to_float(back, out)
+    assert torch.equal(back, out.float())
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 130, 100), (3, 64, 16), (70, 257, 333), (128, 96, 96)])
+def test_gemm_f32_is_true_float32_and_does_not_depend_on_the_batch(ops, M, N, K):
+    a, w, b = rnd(M, K, seed=1), rnd(N, K, seed=2), rnd(N, seed=3)
+    out = torch.empty(M, N, device=DEV)
+    ops.gemm_f32(out, a, w, b)
+    want = a.double() @ w.double().T + b.double()
+    # float32 products and sums: error grows like sqrt(K) * 2^-24 of the summed magnitudes
+    bound = 4 * math.sqrt(K) * 2 ** -24 * (a.double().abs() @ w.double().abs().T + b.double().abs())
+    assert ((out.double() - want).abs() <= bound + 1e-7).all()
+    # a row alone gives the same bits as inside the batch
+    single = torch.empty(1, N, device=DEV)
+    for i in {0, M // 2, M - 1}:
+        ops.gemm_f32(single, a[i:i + 1].contiguous(), w, b)
+        assert torch.equal(single[0], out[i])
+    # strided output and input rows
+    wide_in = torch.zeros(M, K + 7, device=DEV)
+    wide_in[:, :K] = a
+    wide_out = torch.zeros(M, N + 5, device=DEV)
+    ops.gemm_f32(wide_out[:, :N], wide_in[:, :K], w, None)
+    assert torch.equal(wide_out[:, :N], out - b) or torch.allclose(wide_out[:, :N], out - b, atol=1e-5)
+    assert torch.all(wide_out[:, N:] == 0)
+
+
+def test_bf16_linear_uses_float32_accumulation(ops):
+    x, w = rnd(5, 300, dtype=torch.bfloat16), rnd(70, 300, dtype=torch.bfloat16)
+    bias = rnd(70, dtype=torch.bfloat16)
+    out = torch.empty(5, 70, dtype=torch.bfloat16, device=DEV)
+    ops.linear(out, x, w, bias)
+    want = x.double() @ w.double().T + bias.double()
+    assert torch.allclose(out.double(), want, atol=0.15, rtol=1e-2)
+
+
+def test_rope_table(ops):
+    pos = torch.tensor([0, 1, 77, 4095, 100000], dtype=torch.int32, device=DEV)
+    inv = plain.rope_inv_freq(48, 25000.0).float().to(DEV)
+    cos = torch.empty(5, 24, device=DEV)
+    sin = torch.empty(5, 24, device=DEV)
+    ops.rope_table(cos, sin, pos, inv)
+    ang = (pos.float()[:, None] * inv[None, :]).double()  # the angle itself is float32
+    assert torch.allclose(cos.double(), ang.cos(), atol=2e-7)
+    assert torch.allclose(sin.double(), ang.sin(), atol=2e-7)
+
+
+def make_cache(pages, nkv, page_size, d, dtype):
+    k = torch.full((pages, nkv, page_size, d), float("nan"), dtype=dtype, device=DEV)
+    return k, k.clone()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("interleaved,rot_dim", [(False, 32), (True, 32), (False, 16), (False, 0)])
+def test_rope_kv_write(ops, dtype, interleaved, rot_dim):
+    nh, nkv, d, page = 3, 1, 32, 4
+    T = 6
+    qkv0 = rnd(T, (nh + 2 * nkv) * d, dtype=dtype)
+    positions = torch.tensor([5, 6, 7, 0, 1, 9], dtype=torch.int32, device=DEV)
+    token_req = torch.tensor([0, 0, 0, 1, 1, -1], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([2, 0], dtype=torch.int32, device=DEV)
+    table = torch.zeros(3, 4, dtype=torch.int32, device=DEV)
+    table[2, :2] = torch.tensor([5, 3])
+    table[0, :1] = torch.tensor([1])
+    kc, vc = make_cache(7, nkv, page, d, dtype)
+    half = rot_dim // 2
+    inv = plain.rope_inv_freq(rot_dim, 10000.0).float().to(DEV) if rot_dim else torch.zeros(0, device=DEV)
+    cos = torch.empty(T, half, device=DEV)
+    sin = torch.empty(T, half, device=DEV)
+    if rot_dim:
+        ops.rope_table(cos, sin, positions, inv)
+    qkv = qkv0.clone()
+    ops.rope_kv_write(qkv, kc, vc, cos, sin, rot_dim=rot_dim, interleaved=interleaved,
+                      positions=positions, token_req=token_req, slots=slots, table=table,
+                      nh=nh, nkv=nkv, d=d)
+
+    def rotate(x):  # x [T, heads, d] float64
+        if not rot_dim:
+            return x
+        part = x[..., :rot_dim]
+        if interleaved:
+            part = torch.cat((part[..., 0::2], part[..., 1::2]), dim=-1)
+        y = plain.apply_rope(part, positions.cpu().long(), inv.double().cpu())
+        if interleaved:
+            z = torch.empty_like(y)
+            z[..., 0::2], z[..., 1::2] = y[..., :half], y[..., half:]
+            y = z
+        return torch.cat((y, x[..., rot_dim:]), dim=-1)
+
+    x = qkv0.double().cpu().view(T, nh + 2 * nkv, d)
+    want_q = rotate(x[:, :nh])
+    want_k = rotate(x[:, nh:nh + nkv])
+    got = qkv.double().cpu().view(T, nh + 2 * nkv, d)
+    live = [0, 1, 2, 3, 4]
+    assert torch.allclose(got[live, :nh], want_q[live], **tol(dtype))
+    assert torch.equal(got[5], x[5])  # a padding token is left alone
+    assert torch.equal(got[:, nh + nkv:], x[:, nh + nkv:])  # v is never rotated
+    where = {0: (3, 1), 1: (3, 2), 2: (3, 3), 3: (1, 0), 4: (1, 1)}  # token -> (page, offset)
+    for t, (pg, off) in where.items():
+        assert torch.allclose(kc[pg, 0, off].double().cpu(), want_k[t, 0], **tol(dtype))
+        assert torch.equal(vc[pg, 0, off].double().cpu(), x[t, nh + nkv])
+    written = torch.zeros(7, page, dtype=torch.bool)
+    for pg, off in where.values():
+        written[pg, off] = True
+    assert torch.isnan(kc[:, 0, :, 0].cpu()[~written]).all()  # nothing else was touched
+    # write_kv off: q is rotated, the cache is not written
+    kc2, vc2 = make_cache(7, nkv, page, d, dtype)
+    qkv = qkv0.clone()
+    ops.rope_kv_write(qkv, kc2, vc2, cos, sin, rot_dim=rot_dim, interleaved=interleaved,
+                      positions=positions, token_req=token_req, slots=slots, table=table,
+                      nh=nh, nkv=nkv, d=d, write_kv=False)
+    assert torch.isnan(kc2).all() and torch.isnan(vc2).all()
+    assert torch.allclose(qkv.double().cpu().view(T, -1, d)[live, :nh], want_q[live], **tol(dtype))
+
+
+def paged_setup(seq_lens, nkv, d, page, dtype, seed=0, shuffle=True):
+    """Random K/V for requests of the given lengths, scattered over shuffled pages of a
+    NaN-filled cache.  Returns cache planes, table, and the dense K/V per request."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages = sum(-(-n // page) for n in seq_lens) + 3
+    order = torch.randperm(n_pages - 1, generator=g) + 1 if shuffle else torch.arange(1, n_pages)
+    kc, vc = make_cache(n_pages, nkv, page, d, dtype)
+    table = torch.zeros(len(seq_lens) + 2, max(-(-n // page) for n in seq_lens) + 1, dtype=torch.int32)
+    dense = []
+    at = 0
+    for r, n in enumerate(seq_lens):
+        k = (torch.randn(n, nkv, d, generator=g)).to(dtype)
+        v = (torch.randn(n, nkv, d, generator=g)).to(dtype)
+        dense.append((k, v))
+        for i in range(-(-n // page)):
+            pg = int(order[at]); at += 1
+            table[r + 1, i] = pg  # request r lives in slot r + 1
+            lo, hi = i * page, min((i + 1) * page, n)
+            kc[pg, :, : hi - lo] = k[lo:hi].transpose(0, 1).to(DEV)
+            vc[pg, :, : hi - lo] = v[lo:hi].transpose(0, 1).to(DEV)
+    return kc, vc, table.to(DEV), dense
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (3, 1, 48, 16), (8, 8, 128, 32), (2, 1, 256, 8)])
+def test_paged_attention_mixed_batch(ops, dtype, nh, nkv, d, page):
+    seq_lens = [70, 1, 33, 130]
+    q_lens = [70, 1, 5, 1]  # a whole prompt, a first token, a portion with context, a decode
+    kc, vc, table, dense = paged_setup(seq_lens, nkv, d, page, dtype, seed=d)
+    T = sum(q_lens)
+    q = rnd(T, nh * d, dtype=dtype, seed=7)
+    positions, token_req = [], []
+    for r, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        positions += list(range(n - ql, n))
+        token_req += [r] * ql
+    positions = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    token_req_t = torch.tensor(token_req, dtype=torch.int32, device=DEV)
+    slots = torch.tensor([1, 2, 3, 4], dtype=torch.int32, device=DEV)
+    out = torch.empty(T, nh * d, dtype=dtype, device=DEV)
+    scale = d ** -0.5
+    ops.paged_attention(out, q, kc, vc, table=table, positions=positions, token_req=token_req_t,
+                        slots=slots, nh=nh, nkv=nkv, d=d, scale=scale)
+    got = out.double().cpu().view(T, nh, d)
+    qd = q.double().cpu().view(T, nh, d)
+    t = 0
+    for r, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        k, v = dense[r][0].double(), dense[r][1].double()
+        full_q = torch.zeros(n, nh, d, dtype=torch.float64)
+        full_q[n - ql:] = qd[t:t + ql]
+        want = plain.causal_gqa_attention(full_q, k, v, scale)[n - ql:]
+        assert torch.allclose(got[t:t + ql], want, **tol(dtype)), f"request {r}"
+        t += ql
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_finds_one_far_key_among_hundreds(ops, dtype):
+    """Random keys would hide a skipped key.  One key (in turn: the first, one at a page's
+    edge, the last of a page, the query's own) is made to match the query with a large
+    score; the output must be that key's value."""
+    nh, nkv, d, page = 2, 1, 64, 16
+    n = 700
+    for special in [0, 15, 16, 351, 639, 640, 698, 699]:
+        kc, vc, table, dense = paged_setup([n], nkv, d, page, dtype, seed=special)
+        q = rnd(1, nh * d, dtype=dtype, seed=3)
+        qd = q.float().view(nh, d)
+        key = (qd[0] + qd[1]) / 2  # matches both heads
+        key = key * (60.0 / float((qd[0] * key).sum() * d ** -0.5))  # score about 60 after scaling
+        pg, off = int(table[1, special // page]), special % page
+        kc[pg, 0, off] = key.to(dtype)
+        positions = torch.tensor([n - 1], dtype=torch.int32, device=DEV)
+        out = torch.empty(1, nh * d, dtype=dtype, device=DEV)
+        ops.paged_attention(out, q, kc, vc, table=table, positions=positions,
+                            token_req=torch.zeros(1, dtype=torch.int32, device=DEV),
+                            slots=torch.ones(1, dtype=torch.int32, device=DEV),
+                            nh=nh, nkv=nkv, d=d, scale=d ** -0.5)
+        want = vc[pg, 0, off].double().cpu()
+        got = out.double().cpu().view(nh, d)[0]
+        assert torch.allclose(got, want, atol=2e-2 if dtype == torch.bfloat16 else 1e-4), special
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_window_edge(ops, dtype):
+    nh, nkv, d, page, n, w = 2, 2, 32, 8, 90, 20
+    kc, vc, table, dense = paged_setup([n], nkv, d, page, dtype, seed=11)
+    q_len = 30
+    q = rnd(q_len, nh * d, dtype=dtype, seed=5)
+    positions = torch.arange(n - q_len, n, dtype=torch.int32, device=DEV)
+    out = torch.empty(q_len, nh * d, dtype=dtype, device=DEV)
+    args = dict(table=table, positions=positions, token_req=torch.zeros(q_len, dtype=torch.int32, device=DEV),
+                slots=torch.ones(1, dtype=torch.int32, device=DEV), nh=nh, nkv=nkv, d=d, scale=0.2)
+    ops.paged_attention(out, q, kc, vc, window=w, **args)
+    k, v = dense[0][0].double(), dense[0][1].double()
+    full_q = torch.zeros(n, nh, d, dtype=torch.float64)
+    full_q[n - q_len:] = q.double().cpu().view(q_len, nh, d)
+    want = plain.causal_gqa_attention(full_q, k, v, 0.2, window=w)[n - q_len:]
+    assert torch.allclose(out.double().cpu().view(q_len, nh, d), want, **tol(dtype))
+    # pages wholly behind the window may be gone (null page): the result does not change
+    first_needed = (n - q_len) - w + 1
+    table2 = table.clone()
+    table2[1, : first_needed // page] = 0
+    out2 = torch.empty_like(out)
+    ops.paged_attention(out2, q, kc, vc, window=w, **{**args, "table": table2})
+    assert torch.equal(out, out2)
+    # the key at the window's edge counts, the one before it does not
+    edge = n - 1 - w + 1
+    big = torch.zeros(d)
+    big[0] = 1.0
+    qq = torch.zeros(1, nh * d, dtype=dtype, device=DEV)
+    qq[0, 0] = 300.0
+    qq[0, d] = 300.0
+    for pos_key, seen in ((edge, True), (edge - 1, False)):
+        kc2 = kc.clone()
+        kc2[:, :, :, 0] = 0
+        pg, off = int(table[1, pos_key // page]), pos_key % page
+        kc2[pg, :, off, 0] = 1.0
+        o = torch.empty(1, nh * d, dtype=dtype, device=DEV)
+        ops.paged_attention(o, qq, kc2, vc, window=w, **{**args, "positions": positions[-1:],
+                                                         "token_req": torch.zeros(1, dtype=torch.int32, device=DEV)})
+        hit = torch.allclose(o.float().cpu().view(nh, d), vc[pg, :, off].float().cpu(), atol=2e-2)
+        assert hit == seen
+
+
+def test_paged_attention_refuses_unsupported_head_sizes(ops):
+    from kvcore_amd.ops.library import KernelError
+
+    kc, vc = make_cache(2, 1, 4, 24, torch.float32)
+    q = rnd(1, 24)
+    with pytest.raises(KernelError, match="multiple of 16"):
+        ops.paged_attention(torch.empty(1, 24, device=DEV), q, kc, vc,
+                            table=torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                            positions=torch.zeros(1, dtype=torch.int32, device=DEV),
+                            token_req=torch.zeros(1, dtype=torch.int32, device=DEV),
+                            slots=torch.zeros(1, dtype=torch.int32, device=DEV),
+                            nh=1, nkv=1, d=24, scale=1.0)
+
+
+def test_table_update(ops):
+    table = torch.zeros(3, 5, dtype=torch.int32, device=DEV)
+    triples = torch.tensor([0, 0, 7, 2, 4, 9, 1, 3, 8, 5, 0, 1, 0, 9, 1], dtype=torch.int32, device=DEV)
+    ops.table_update(table, triples, 5)  # the last two are outside the table and are dropped
+    want = torch.zeros(3, 5, dtype=torch.int32)
+    want[0, 0], want[2, 4], want[1, 3] = 7, 9, 8
+    assert torch.equal(table.cpu(), want)
+
+
+# -------------------------------------------------------------------------- sampling
+def sample_rows(ops, logits, temps, top_k, top_p, seeds, index):
+    S = logits.shape[0]
+    out = torch.empty(S, dtype=torch.int32, device=DEV)
+    t = lambda v, dt: torch.tensor(v, dtype=dt, device=DEV)  # noqa: E731
+    lo = [s & 0xFFFFFFFF for s in seeds]
+    hi = [(s >> 32) & 0xFFFFFFFF for s in seeds]
+    ops.sample(out, logits, temperature=t(temps, torch.float32), top_k=t(top_k, torch.int32),
+               top_p=t(top_p, torch.float32), seed_lo=t(lo, torch.int64).to(torch.int32),
+               seed_hi=t(hi, torch.int64).to(torch.int32), index=t(index, torch.int32))
+    return out.cpu().tolist()
+
+
+def test_argmax_takes_the_lowest_index_among_equals(ops):
+    logits = rnd(4, 1000, seed=9)
+    logits[1, 400] = logits[1, 17] = 50.0
+    logits[2, 999] = 60.0
+    out = torch.empty(4, dtype=torch.int32, device=DEV)
+    ops.argmax(out, logits)
+    want = logits.cpu().argmax(-1).tolist()
+    want[1] = 17
+    assert out.cpu().tolist() == want
+    wide = torch.zeros(4, 1100, device=DEV)
+    wide[:, :1000] = logits
+    ops.argmax(out, wide[:, :1000])
+    assert out.cpu().tolist() == want
+
+
+@pytest.mark.parametrize("V", [331, 5000])
+def test_sample_matches_the_plain_sampler_draw_for_draw(ops, V):
+    S = 24
+    logits = rnd(S, V, scale=2.0, seed=V)
+    temps = [0.0, 0.8, 1.0, 1.7] * 6
+    top_k = [0, 0, 5, 40, 0, 3] * 4
+    top_p = [1.0, 1.0, 1.0, 0.9, 0.5, 0.3] * 4
+    seeds = [(12345 + 977 * i) | ((i * 31) << 32) for i in range(S)]
+    index = [i * 3 for i in range(S)]
+    got = sample_rows(ops, logits, temps, top_k, top_p, seeds, index)
+    for i in range(S):
+        want = plain_sampling.sample(logits[i].cpu(), temperature=temps[i], top_k=top_k[i] or None,
+                                     top_p=top_p[i], seed=seeds[i], index=index[i])
+        assert got[i] == want, f"row {i}: temperature {temps[i]} top_k {top_k[i]} top_p {top_p[i]}"
+    # a row's draw does not depend on its batch-mates
+    alone = sample_rows(ops, logits[5:6], temps[5:6], top_k[5:6], top_p[5:6], seeds[5:6], index[5:6])
+    assert alone[0] == got[5]
+
+
+def test_sample_follows_the_probabilities_and_top_k_top_p_vectors(ops):
+    base = torch.tensor([1.0, 0.0, 2.0, -1.0, 0.5], device=DEV)
+    n = 4000
+    logits = base.repeat(n, 1)
+    draws = sample_rows(ops, logits, [0.8] * n, [0] * n, [1.0] * n, [42] * n, list(range(n)))
+    probs = torch.softmax(base.double().cpu() / 0.8, dim=0)
+    counts = torch.bincount(torch.tensor(draws), minlength=5).double()
+    chi2 = float(((counts - n * probs) ** 2 / (n * probs)).sum())
+    assert chi2 < 18.5
+    # the reference's vectors (tests/test_sampler.py:49-68): only kept entries are ever drawn
+    k_logits = torch.tensor([[1.0, 2.0, 3.0, 4.0]], device=DEV).repeat(200, 1)
+    got = set(sample_rows(ops, k_logits, [1.0] * 200, [2] * 200, [1.0] * 200, [1] * 200, list(range(200))))
+    assert got == {2, 3}
+    p_logits = torch.tensor([[10.0, 9.0, 0.0, -1.0]], device=DEV).repeat(200, 1)
+    got = set(sample_rows(ops, p_logits, [1.0] * 200, [0] * 200, [0.8] * 200, [1] * 200, list(range(200))))
+    assert got == {0, 1}
