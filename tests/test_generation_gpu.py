@@ -1,0 +1,166 @@
+"""Generation through the Python entry point and the command line, against the plain
+implementation: greedy (tiny A's workload), seeded temperature sampling (tiny B's),
+chunked prefill, preemption when pages run out."""
+
+from __future__ import annotations
+
+import math
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+from tests.helpers import CONFIGS, make_model_dir, random_tokens
+from tests.plain import llama as plain
+from tests.plain import sampling as plain_sampling
+
+pytestmark = pytest.mark.gpu
+REPO = Path(__file__).resolve().parent.parent
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name, (config, page) in CONFIGS.items():
+        folder = make_model_dir(tmp_path_factory.mktemp(f"gen_{name}"), config, seed=21)
+        out[name] = (folder, *plain.load_model_folder(folder), page)
+    return out
+
+
+def make_engine(folder, dtype, page, *, num_pages=None, max_seqs=4, budget=64, partial=4, threshold=0):
+    from kvcore_amd import (CacheConfig, KVCoreConfig, LoadConfig, ModelConfig, SchedulerConfig)
+    from kvcore_amd.engine.llm_engine import LLMEngine
+
+    return LLMEngine(KVCoreConfig(
+        model_config=ModelConfig(model=str(folder), dtype=dtype),
+        load_config=LoadConfig(seed=77),
+        cache_config=CacheConfig(block_size=page, num_gpu_blocks=num_pages),
+        scheduler_config=SchedulerConfig(max_num_seqs=max_seqs, max_num_scheduled_tokens=budget,
+                                         max_num_partial_prefills=partial, max_long_partial_prefills=partial,
+                                         long_prefill_token_threshold=threshold),
+    ))
+
+
+def check_tokens(cfg, weights, prompt, tokens, *, temperature, seed, tol):
+    """Every generated token must be the plain sampler's choice on the plain logits of the
+    same prefix, or tie with it within rounding (``tol`` on the compared scores)."""
+    ids = list(prompt)
+    for index, tok in enumerate(tokens):
+        logits = plain.llama_forward(cfg, weights, ids, dtype=torch.float64)[-1]
+        if temperature < 1e-5:
+            score = logits
+        else:
+            noise = plain_sampling.exponential_noise(seed, index, logits.numel())
+            score = logits / temperature - torch.log(noise)
+        gap = float(score.max() - score[tok])
+        assert gap <= tol, (f"token {index}: engine chose {tok}, plain prefers {int(score.argmax())} "
+                            f"by {gap:.2e}")
+        ids.append(tok)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 4e-2)])
+def test_greedy_generation_through_the_entry_point(folders, dtype, tol):
+    from kvcore_amd import SamplingParams
+    from kvcore_amd.engine.llm_engine import GenerationRequest
+
+    folder, cfg, weights, page = folders["A"]
+    prompts = {f"r{n}": random_tokens(n, 256, seed=n) for n in (7, 16, 33, 50)}
+    engine = make_engine(folder, dtype, page)
+    outs = engine.generate([
+        GenerationRequest(rid, SamplingParams(max_tokens=16, temperature=0.0, ignore_eos=True),
+                          prompt_token_ids=tuple(p)) for rid, p in prompts.items()])
+    assert [o.request_id for o in outs] == list(prompts)
+    for o in outs:
+        assert len(o.output_token_ids) == 16 and o.finish_reason == "length"
+        check_tokens(cfg, weights, prompts[o.request_id], o.output_token_ids, temperature=0.0, seed=0, tol=tol)
+        if dtype == "float32":
+            assert list(o.output_token_ids) == plain.greedy_generate(cfg, weights, prompts[o.request_id], 16)
+    core = engine.engine_core
+    assert core.kv_manager.num_free_pages() == [core.num_pages - 1]  # idle: every page is back
+    assert core.kv_manager.slots.num_free == 4
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 5e-5), ("bfloat16", 6e-2)])
+def test_seeded_temperature_sampling_with_chunked_prefill(folders, dtype, tol):
+    """Tiny B's workload: prompts 1/9/24/40/61, temperature 0.8 with a fixed seed, 32 new
+    tokens, prompts cut into portions of 16."""
+    from kvcore_amd import SamplingParams
+
+    folder, cfg, weights, page = folders["B"]
+    prompts = {f"r{n}": random_tokens(n, 384, seed=100 + n) for n in (1, 9, 24, 40, 61)}
+    engine = make_engine(folder, dtype, page, budget=40, threshold=16)
+    reqs = [dict(request_id=rid, prompt_token_ids=p,
+                 sampling_params=SamplingParams(max_tokens=32, temperature=0.8, seed=1234 + i, ignore_eos=True))
+            for i, (rid, p) in enumerate(prompts.items())]
+    outs = {o.request_id: o for o in engine.generate(reqs)}
+    for i, (rid, p) in enumerate(prompts.items()):
+        toks = outs[rid].output_token_ids
+        assert len(toks) == 32
+        check_tokens(cfg, weights, p, toks, temperature=0.8, seed=1234 + i, tol=tol)
+        assert len(set(toks)) > 8  # fresh noise at every token
+    # the same seeds give the same tokens, whatever the batching
+    again = make_engine(folder, dtype, page, budget=64, max_seqs=2)
+    outs2 = {o.request_id: o for o in again.generate(reqs)}
+    if dtype == "float32":
+        assert all(outs2[r].output_token_ids == outs[r].output_token_ids for r in prompts)
+
+
+def test_generation_survives_running_out_of_pages(folders):
+    """So few pages that running requests must be preempted and recomputed; the outputs are
+    those of an engine with plenty of pages."""
+    from kvcore_amd import SamplingParams
+
+    folder, cfg, weights, page = folders["A"]
+    prompts = {f"r{i}": random_tokens(n, 256, seed=300 + i) for i, n in enumerate((20, 30, 25, 18))}
+    reqs = [dict(request_id=rid, prompt_token_ids=p,
+                 sampling_params=SamplingParams(max_tokens=30, temperature=0.0, ignore_eos=True))
+            for rid, p in prompts.items()]
+    roomy = make_engine(folder, "float32", page)
+    want = {o.request_id: o.output_token_ids for o in roomy.generate(reqs)}
+    tight = make_engine(folder, "float32", page, num_pages=9)  # 8 usable pages of 16 tokens
+    got = {o.request_id: o.output_token_ids for o in tight.generate(reqs)}
+    assert tight.engine_core.scheduler.num_preemptions > 0
+    assert got == want
+    assert tight.engine_core.kv_manager.num_free_pages() == [8]
+    # a request that can never fit is refused at once
+    with pytest.raises(ValueError, match="cache pages"):
+        tight.add_request("big", SamplingParams(max_tokens=100), prompt_token_ids=list(range(100)))
+
+
+def test_stop_token_ends_a_request(folders):
+    from kvcore_amd import SamplingParams
+
+    folder, cfg, weights, page = folders["A"]
+    prompt = random_tokens(12, 256, seed=9)
+    tokens = plain.greedy_generate(cfg, weights, prompt, 8)
+    engine = make_engine(folder, "float32", page)
+    engine.engine_core.stop_token_ids = {tokens[3]}
+    out = engine.generate([dict(request_id="s", prompt_token_ids=prompt,
+                                sampling_params=SamplingParams(max_tokens=8, temperature=0.0))])[0]
+    first = tokens.index(tokens[3])
+    assert list(out.output_token_ids) == tokens[: first + 1] and out.finish_reason == "stop"
+
+
+def test_command_line(folders, tmp_path):
+    folder, cfg, weights, page = folders["A"]
+    cmd = [sys.executable, str(REPO / "bin" / "kvcore_offline_batch"), "--model", str(folder),
+           "--dtype", "float32", "--prompt-lens", "7,16", "--max-tokens", "5", "--seed", "3",
+           "--max-num-seqs", "4", "--max-num-scheduled-tokens", "32", "--num-gpu-blocks", "32",
+           "--ignore-eos", "--log-level", "WARNING", "--log-file", str(tmp_path / "run.log")]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=240)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    text = proc.stdout
+    for section in ("=== Run Metadata ===", "=== Requests ===", "=== Detokenized Outputs ===",
+                    "=== Timing Summary ===", "engine_init_sec=", "generate_sec=", "total_elapsed_sec="):
+        assert section in text
+    assert text.count("finish_reason=length") == 2
+    assert (tmp_path / "run.log").read_text().count("finish_reason=length") == 2
+    import random
+
+    rng = random.Random(3)
+    first_prompt = [rng.randrange(256) for _ in range(7)]
+    line = next(l for l in text.splitlines() if l.startswith("token_ids="))
+    got = [int(x) for x in line.split("=", 1)[1].strip("()").split(",") if x.strip()]
+    assert got == plain.greedy_generate(cfg, weights, first_prompt, 5)
