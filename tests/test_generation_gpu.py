@@ -125,8 +125,9 @@ def test_generation_survives_running_out_of_pages(folders):
     assert got == want
     assert tight.engine_core.kv_manager.num_free_pages() == [8]
     # a request that can never fit is refused at once
+    tiny = make_engine(folder, "float32", page, num_pages=4)  # 3 usable pages hold 48 tokens
     with pytest.raises(ValueError, match="cache pages"):
-        tight.add_request("big", SamplingParams(max_tokens=100), prompt_token_ids=list(range(100)))
+        tiny.add_request("big", SamplingParams(max_tokens=10), prompt_token_ids=list(range(50)))
 
 
 def test_stop_token_ends_a_request(folders):
