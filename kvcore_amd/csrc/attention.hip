@@ -6,7 +6,7 @@
 // tile: each lane scores one key (a float32 dot product over the head in index
 // order), the tile is folded into a running softmax (float32 max, sum and output
 // accumulators), then the lanes split the head's elements to add p_j * V_j in key
-// order.  What a token computes depends on its position, window and cache content
+// order.  K pages are [kv head, page_size, d], V pages [kv head, d, page_size].  What a token computes depends on its position, window and cache content
 // only: not on the batch it is in nor on how its request was cut into steps.
 
 #include <hip/hip_runtime.h>
@@ -48,7 +48,8 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     float scale, int window) {
   __shared__ float q_s[kWavesPerBlock][kMaxHeadDim];
   __shared__ float p_s[kWavesPerBlock][kWave];
-  __shared__ int64_t off_s[kWavesPerBlock][kWave];
+  __shared__ int64_t off_s[kWavesPerBlock][kWave];   // K row of each key of the tile
+  __shared__ int64_t voff_s[kWavesPerBlock][kWave];  // V column of each key of the tile
 
   const int t = blockIdx.x;
   const int wave = threadIdx.x / kWave;
@@ -86,12 +87,13 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     const int key = tile + lane;
     const bool valid = key <= pos;
     float s = -INFINITY;
-    int64_t off = -1;
+    int64_t off = -1, voff = -1;
     if (valid) {
       const int page = row[key / page_size];
       if (page > 0 && page < num_pages) {
         off = static_cast<int64_t>(page) * page_elems + head_off +
               static_cast<int64_t>(key % page_size) * d;
+        voff = static_cast<int64_t>(page) * page_elems + head_off + key % page_size;
         const T* kr = k_cache + off;
         float dot = 0.f;
         for (int i = 0; i < d; i += VN) {
@@ -113,19 +115,20 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     __syncthreads();
     p_s[wave][lane] = p;
     off_s[wave][lane] = off;
+    voff_s[wave][lane] = voff;
     __syncthreads();
     const int n_keys = (pos - tile + 1 < kWave) ? pos - tile + 1 : kWave;
 #pragma unroll
     for (int i = 0; i < kMaxHeadDim / kWave; ++i) acc[i] *= alpha;
     for (int j = 0; j < n_keys; ++j) {
-      const int64_t voff = off_s[wave][j];
-      if (voff < 0) continue;
+      const int64_t vo = voff_s[wave][j];
+      if (vo < 0) continue;
       const float pj = p_s[wave][j];
-      const T* vr = v_cache + voff;
+      const T* vr = v_cache + vo;  // element e of this key is at vr[e * page_size]
 #pragma unroll
       for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
         const int e = lane + i * kWave;
-        if (e < d) acc[i] = fmaf(pj, to_float(vr[e]), acc[i]);
+        if (e < d) acc[i] = fmaf(pj, to_float(vr[static_cast<int64_t>(e) * page_size]), acc[i]);
       }
     }
   }

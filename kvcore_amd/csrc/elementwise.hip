@@ -269,12 +269,16 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
   const int half = rot_dim / 2;
   T* row = qkv + static_cast<int64_t>(t) * (nh + 2 * nkv) * d;
 
-  int64_t cache_base = -1;  // element offset of [page, kv head 0, pos % page_size, 0]
+  // K pages are [kv head, page_size, d]; V pages are [kv head, d, page_size] (keys contiguous)
+  int64_t cache_base = -1;  // element offset of K[page, kv head 0, pos % page_size, 0]
+  int64_t v_base = -1;      // element offset of V[page, kv head 0, 0, pos % page_size]
   if (write_kv) {
     const int slot = slots[req];
     const int page = table[static_cast<int64_t>(slot) * table_stride + pos / page_size];
-    if (page > 0 && page < num_pages)
+    if (page > 0 && page < num_pages) {
       cache_base = (static_cast<int64_t>(page) * nkv * page_size + pos % page_size) * d;
+      v_base = static_cast<int64_t>(page) * nkv * page_size * d + pos % page_size;
+    }
   }
   const int64_t head_step = static_cast<int64_t>(page_size) * d;  // between kv heads in a page
 
@@ -316,7 +320,8 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
   for (int w = threadIdx.x; w < nkv * d; w += blockDim.x) {
     const int head = w / d;
     const int i = w - head * d;
-    v_cache[cache_base + head * head_step + i] = row[static_cast<int64_t>(nh + nkv + head) * d + i];
+    v_cache[v_base + head * head_step + static_cast<int64_t>(i) * page_size] =
+        row[static_cast<int64_t>(nh + nkv + head) * d + i];
   }
 }
 

@@ -52,7 +52,8 @@ int kvc_rope_table(float* cos_out, float* sin_out, const int32_t* positions,
 // place (pairs (j, j+rot_dim/2), or (2j, 2j+1) when interleaved), then, when write_kv is
 // set, stores the rotated k and the v of token t at its page slot:
 //   slot row  = slots[token_req[t]], page = table[row, pos / page_size],
-//   cache[page, kv_head, pos % page_size, :].
+//   k_cache[page, kv_head, pos % page_size, :] and v_cache[page, kv_head, :, pos % page_size]
+//   (V pages keep the keys contiguous: the layout the matrix cores read).
 // Tokens with token_req < 0 are left alone.
 int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_tab,
                       const float* sin_tab, int rot_dim, int interleaved,
@@ -68,6 +69,17 @@ int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* 
                         const int32_t* positions, const int32_t* token_req,
                         const int32_t* slots, int T, int nh, int nkv, int d, int page_size,
                         int num_pages, float scale, int window, int dtype, kvc_stream stream);
+
+// The same attention for bfloat16 on the matrix cores, one wave per (token, kv head,
+// split): meant for steps of single tokens.  nsplit > 1 needs part_o [T, nh, nsplit, d]
+// and part_ml [T, nh, nsplit, 2] float32.  kvc_decode_attention_supported tells whether
+// a shape is served (else use kvc_paged_attention).
+int kvc_decode_attention_supported(int nh, int nkv, int d, int page_size, int dtype);
+int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* q, int64_t q_stride,
+                         const void* k_cache, const void* v_cache, const int32_t* table,
+                         int table_stride, const int32_t* positions, const int32_t* token_req,
+                         const int32_t* slots, int T, int nh, int nkv, int d, int page_size,
+                         int num_pages, float scale, int window, int nsplit, kvc_stream stream);
 
 // C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) in float32 with float32 products and sums;
 // each element is one running sum over k = 0..K-1, whatever M is.

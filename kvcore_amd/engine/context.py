@@ -32,8 +32,8 @@ class LayerCall:
 
 @dataclass
 class CacheGroupView:
-    """Device side of one cache group: ``kv`` is ``[planes, 2, pages, kv_heads,
-    page_size, head_dim]``; ``table`` is ``[max_seqs, max_pages_per_seq]`` int32, row =
+    """Device side of one cache group: ``kv`` is the storage ``[planes, 2, pages, kv_heads,
+    page_size, head_dim]`` (index 0 keys, 1 values; see ``planes`` for the values' layout); ``table`` is ``[max_seqs, max_pages_per_seq]`` int32, row =
     request slot, entry = page id (0 is the null page)."""
 
     kv: torch.Tensor
@@ -42,7 +42,16 @@ class CacheGroupView:
     window: int = 0
 
     def planes(self, cache_index: int) -> tuple[torch.Tensor, torch.Tensor]:
-        return self.kv[cache_index, 0], self.kv[cache_index, 1]
+        """K plane ``[pages, kv_heads, page_size, head_dim]`` and V plane ``[pages, kv_heads,
+        head_dim, page_size]`` (a V page keeps its keys contiguous) of one cache index."""
+        views = self.__dict__.setdefault("_plane_views", {})
+        got = views.get(cache_index)
+        if got is None:
+            k = self.kv[cache_index, 0]
+            pages, heads, page_size, d = k.shape
+            got = (k, self.kv[cache_index, 1].view(pages, heads, d, page_size))
+            views[cache_index] = got
+        return got
 
 
 class StepBuffers:

@@ -39,6 +39,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_rope_table": [P, P, P, P, I, I, P],
         "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
         "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "kvc_decode_attention_supported": [I, I, I, I, I],
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
         "kvc_table_update": [P, I, I, P, I, P],
         "kvc_argmax": [P, P, I, I, L, P],
@@ -188,13 +190,12 @@ def rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                   cos: torch.Tensor, sin: torch.Tensor, *, rot_dim: int, interleaved: bool,
                   positions: torch.Tensor, token_req: torch.Tensor, slots: torch.Tensor,
                   table: torch.Tensor, nh: int, nkv: int, d: int, write_kv: bool = True) -> None:
-    """``k_cache``/``v_cache`` are ``[pages, nkv, page_size, d]`` of the dtype of ``qkv``."""
+    """``k_cache`` is ``[pages, nkv, page_size, d]``, ``v_cache`` ``[pages, nkv, d, page_size]``,
+    both of the dtype of ``qkv``."""
     T = qkv.shape[0]
     if qkv.shape != (T, (nh + 2 * nkv) * d):
         raise KernelError(f"rope_kv_write: qkv shape {tuple(qkv.shape)} does not fit heads")
-    num_pages, ckv, page_size, cd = k_cache.shape
-    if (ckv, cd) != (nkv, d) or v_cache.shape != k_cache.shape:
-        raise KernelError("rope_kv_write: cache shape does not fit heads")
+    num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "rope_kv_write")
     if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
         raise KernelError("rope_kv_write: cache dtype differs from qkv")
     if cos.shape[0] < T or cos.shape[1] != rot_dim // 2 or sin.shape != cos.shape:
@@ -220,9 +221,9 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         raise KernelError("paged_attention: out must be contiguous [T, nh*d]")
     if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or q.dtype != out.dtype:
         raise KernelError("paged_attention: q does not fit")
-    num_pages, ckv, page_size, cd = k_cache.shape
-    if (ckv, cd) != (nkv, d) or v_cache.shape != k_cache.shape or k_cache.dtype != out.dtype:
-        raise KernelError("paged_attention: cache does not fit heads or dtype")
+    num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "paged_attention")
+    if k_cache.dtype != out.dtype:
+        raise KernelError("paged_attention: cache dtype differs from the queries'")
     if positions.numel() < T or token_req.numel() < T:
         raise KernelError("paged_attention: per-token arrays too short")
     _check(load().kvc_paged_attention(
@@ -231,6 +232,55 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
         _dev(slots, "slots", torch.int32), T, nh, nkv, d, page_size, num_pages, float(scale),
         int(window), _code(out, "out"), _stream()), "kvc_paged_attention")
+
+
+def decode_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype: torch.dtype) -> bool:
+    return bool(load().kvc_decode_attention_supported(nh, nkv, d, page_size, DTYPE_CODE.get(dtype, -1)))
+
+
+def decode_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     *, table: torch.Tensor, positions: torch.Tensor, token_req: torch.Tensor,
+                     slots: torch.Tensor, nh: int, nkv: int, d: int, scale: float, window: int = 0,
+                     nsplit: int = 1, part_o: torch.Tensor | None = None,
+                     part_ml: torch.Tensor | None = None) -> None:
+    """bfloat16 attention of single tokens on the matrix cores (see the C header).  ``part_o``
+    and ``part_ml`` are float32 workspaces of at least ``T*nh*nsplit*d`` and ``T*nh*nsplit*2``
+    elements when ``nsplit > 1``."""
+    T = out.shape[0]
+    if out.shape != (T, nh * d) or not out.is_contiguous() or out.dtype != torch.bfloat16:
+        raise KernelError("decode_attention: out must be contiguous bfloat16 [T, nh*d]")
+    if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or q.dtype != out.dtype:
+        raise KernelError("decode_attention: q does not fit")
+    num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "decode_attention")
+    if k_cache.dtype != out.dtype:
+        raise KernelError("decode_attention: cache dtype differs from the queries'")
+    if positions.numel() < T or token_req.numel() < T:
+        raise KernelError("decode_attention: per-token arrays too short")
+    po = pm = None
+    if nsplit > 1:
+        if part_o is None or part_ml is None or part_o.numel() < T * nh * nsplit * d \
+                or part_ml.numel() < T * nh * nsplit * 2:
+            raise KernelError("decode_attention: workspace missing or too small")
+        po, pm = _dev(part_o, "part_o", torch.float32), _dev(part_ml, "part_ml", torch.float32)
+    _check(load().kvc_decode_attention(
+        out.data_ptr(), po, pm, q.data_ptr(), q.stride(0), _dev(k_cache, "k_cache"),
+        _dev(v_cache, "v_cache"), _dev(table, "table", torch.int32), table.shape[1],
+        _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
+        _dev(slots, "slots", torch.int32), T, nh, nkv, d, page_size, num_pages, float(scale),
+        int(window), int(nsplit), _stream()), "kvc_decode_attention")
+
+
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int, who: str) -> tuple[int, int]:
+    """K pages are ``[pages, nkv, page_size, d]``, V pages ``[pages, nkv, d, page_size]``."""
+    if k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise KernelError(f"{who}: cache planes must be 4-D")
+    num_pages, ckv, page_size, cd = k_cache.shape
+    if (ckv, cd) != (nkv, d) or tuple(v_cache.shape) != (num_pages, nkv, d, page_size):
+        raise KernelError(f"{who}: cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
+                          f"{nkv} kv heads of {d}")
+    if k_cache.dtype != v_cache.dtype:
+        raise KernelError(f"{who}: K and V planes differ in dtype")
+    return num_pages, page_size
 
 
 def gemm_f32(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None) -> None:

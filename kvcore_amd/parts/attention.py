@@ -15,6 +15,18 @@ from kvcore_amd.ops import library as ops
 from .base import CacheNeed, Mixer, ParamSource, ParamSpec, PositionEncoding, register_mixer
 
 
+DECODE_TARGET_WAVES = 2048  # enough single-wave blocks to keep 256 compute units fed
+DECODE_MAX_SPLITS = 32
+
+
+def decode_splits(num_tokens: int, num_kv_heads: int, max_seq_len: int) -> int:
+    """Into how many parts each request's key range is cut for the decode kernel: enough
+    that tokens x kv heads x parts fills the chip, never more than there are 16-key blocks."""
+    want = DECODE_TARGET_WAVES // max(num_tokens * num_kv_heads, 1)
+    blocks = -(-max_seq_len // 16)
+    return max(1, min(want, DECODE_MAX_SPLITS, blocks))
+
+
 class PagedAttention(Mixer):
     """``scale`` is a parameter (the reference fixes ``head_dim ** -0.5`` at
     llama3.py:60); ``window`` 0 attends to every earlier token."""
@@ -78,10 +90,23 @@ class PagedAttention(Mixer):
                           d=self.head_dim, write_kv=call.write_cache)
 
         attn = ctx.buf("attn_out", self.q_size)
-        ops.paged_attention(attn, qkv, k_cache, v_cache, table=group.table, positions=ctx.positions,
-                            token_req=ctx.token_req, slots=ctx.slots, nh=self.num_heads,
-                            nkv=self.num_kv_heads, d=self.head_dim, scale=self.scale,
-                            window=self.window)
+        common = dict(table=group.table, positions=ctx.positions, token_req=ctx.token_req,
+                      slots=ctx.slots, nh=self.num_heads, nkv=self.num_kv_heads, d=self.head_dim,
+                      scale=self.scale, window=self.window)
+        if ctx.max_query_len == 1 and ops.decode_attention_supported(
+                self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
+            # single tokens: one wave per (token, kv head, split) on the matrix cores
+            T = ctx.num_tokens
+            nsplit = decode_splits(T, self.num_kv_heads, ctx.max_seq_len)
+            part_o = part_ml = None
+            if nsplit > 1:
+                part_o = ctx.buffers.get("attn_part_o", T * self.num_heads * nsplit, self.head_dim,
+                                         torch.float32)
+                part_ml = ctx.buffers.get("attn_part_ml", T * self.num_heads * nsplit, 2, torch.float32)
+            ops.decode_attention(attn, qkv, k_cache, v_cache, nsplit=nsplit, part_o=part_o,
+                                 part_ml=part_ml, **common)
+        else:
+            ops.paged_attention(attn, qkv, k_cache, v_cache, **common)
         out = ctx.buf("mixer_out", self.hidden_size)
         ops.linear(out, attn, p["o_proj.weight"], p.get("o_proj.bias"))
         return out

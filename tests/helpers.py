@@ -1,6 +1,6 @@
 """Tiny configurations and helpers shared by the tests.
 
-The three configurations differ in every size and option: layer count, width, head
+The first three configurations differ in every size and option: layer count, width, head
 counts and grouping (2:1, 3:1 multi-query, 1:1), head size (16, 32, 48), feed-forward
 width, vocabulary (a power of two, a multiple of 128, an odd number), rope base and
 scaling, tied or untied head, norm eps, biases.
@@ -44,7 +44,21 @@ TINY_C = {
 }
 TINY_C_PAGE = 32
 
-CONFIGS = {"A": (TINY_A, TINY_A_PAGE), "B": (TINY_B, TINY_B_PAGE), "C": (TINY_C, TINY_C_PAGE)}
+# head size 64, four query heads per kv head, pages of 16: the shape class that the
+# matrix-core attention kernels serve in bfloat16 (the other three run the general kernel)
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 2, "hidden_size": 128, "num_attention_heads": 8, "num_key_value_heads": 2,
+    "head_dim": 64, "intermediate_size": 192, "vocab_size": 512, "rope_theta": 1000000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 2.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 8.0, "original_max_position_embeddings": 128},
+    "tie_word_embeddings": False, "rms_norm_eps": 1e-5, "max_position_embeddings": 1024,
+    "hidden_act": "silu",
+}
+TINY_D_PAGE = 16
+
+CONFIGS = {"A": (TINY_A, TINY_A_PAGE), "B": (TINY_B, TINY_B_PAGE), "C": (TINY_C, TINY_C_PAGE),
+           "D": (TINY_D, TINY_D_PAGE)}
 
 
 def make_model_dir(folder: Path, config: dict, seed: int, dtype=torch.bfloat16, bias_std: float = 0.05) -> Path:

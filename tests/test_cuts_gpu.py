@@ -82,12 +82,12 @@ def compare(got, expect_by_id, dtype):
                 f"(engine {row[worst]:.6f}, plain {ref[worst]:.6f})")
 
 
-PROMPT_LENS = {"A": [7, 16, 33, 50], "B": [1, 9, 24, 40, 61], "C": [5, 32, 47, 90]}
+PROMPT_LENS = {"A": [7, 16, 33, 50], "B": [1, 9, 24, 40, 61], "C": [5, 32, 47, 90], "D": [3, 31, 64, 150]}
 EXTRA = 34  # tokens after the prompt, so that 32 of them can be decoded one by one
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_whole_requests_alone(models, name, dtype):
     folder, cfg, weights, page = models[name]
     for i, n in enumerate(PROMPT_LENS[name]):
@@ -100,7 +100,7 @@ def test_whole_requests_alone(models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_prefill_then_decode_one_by_one(models, name, dtype):
     folder, cfg, weights, page = models[name]
     for i, n in enumerate(PROMPT_LENS[name]):
@@ -117,7 +117,7 @@ def test_prefill_then_decode_one_by_one(models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_portions_of_changing_size(models, name, dtype):
     folder, cfg, weights, page = models[name]
     sizes = [16, 7, 2, 5, 13, 2, 3, 9, 2, 11, 4, 2]
@@ -179,7 +179,7 @@ def mixed_trace(token_lists, seed):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_mixed_batches_with_page_reuse(models, name, dtype):
     folder, cfg, weights, page = models[name]
     base = PROMPT_LENS[name]

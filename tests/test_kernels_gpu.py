@@ -140,8 +140,9 @@ def test_rope_table(ops):
 
 
 def make_cache(pages, nkv, page_size, d, dtype):
+    """K pages [pages, nkv, page_size, d]; V pages [pages, nkv, d, page_size]; all NaN."""
     k = torch.full((pages, nkv, page_size, d), float("nan"), dtype=dtype, device=DEV)
-    return k, k.clone()
+    return k, k.clone().view(pages, nkv, d, page_size)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -192,7 +193,7 @@ def test_rope_kv_write(ops, dtype, interleaved, rot_dim):
     where = {0: (3, 1), 1: (3, 2), 2: (3, 3), 3: (1, 0), 4: (1, 1)}  # token -> (page, offset)
     for t, (pg, off) in where.items():
         assert torch.allclose(kc[pg, 0, off].double().cpu(), want_k[t, 0], **tol(dtype))
-        assert torch.equal(vc[pg, 0, off].double().cpu(), x[t, nh + nkv])
+        assert torch.equal(vc[pg, 0, :, off].double().cpu(), x[t, nh + nkv])
     written = torch.zeros(7, page, dtype=torch.bool)
     for pg, off in where.values():
         written[pg, off] = True
@@ -226,7 +227,7 @@ def paged_setup(seq_lens, nkv, d, page, dtype, seed=0, shuffle=True):
             table[r + 1, i] = pg  # request r lives in slot r + 1
             lo, hi = i * page, min((i + 1) * page, n)
             kc[pg, :, : hi - lo] = k[lo:hi].transpose(0, 1).to(DEV)
-            vc[pg, :, : hi - lo] = v[lo:hi].transpose(0, 1).to(DEV)
+            vc[pg, :, :, : hi - lo] = v[lo:hi].permute(1, 2, 0).to(DEV)
     return kc, vc, table.to(DEV), dense
 
 
@@ -282,7 +283,7 @@ def test_paged_attention_finds_one_far_key_among_hundreds(ops, dtype):
                             token_req=torch.zeros(1, dtype=torch.int32, device=DEV),
                             slots=torch.ones(1, dtype=torch.int32, device=DEV),
                             nh=nh, nkv=nkv, d=d, scale=d ** -0.5)
-        want = vc[pg, 0, off].double().cpu()
+        want = vc[pg, 0, :, off].double().cpu()
         got = out.double().cpu().view(nh, d)[0]
         assert torch.allclose(got, want, atol=2e-2 if dtype == torch.bfloat16 else 1e-4), special
 
@@ -325,8 +326,89 @@ def test_paged_attention_window_edge(ops, dtype):
         o = torch.empty(1, nh * d, dtype=dtype, device=DEV)
         ops.paged_attention(o, qq, kc2, vc, window=w, **{**args, "positions": positions[-1:],
                                                          "token_req": torch.zeros(1, dtype=torch.int32, device=DEV)})
-        hit = torch.allclose(o.float().cpu().view(nh, d), vc[pg, :, off].float().cpu(), atol=2e-2)
+        hit = torch.allclose(o.float().cpu().view(nh, d), vc[pg, :, :, off].float().cpu(), atol=2e-2)
         assert hit == seen
+
+
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 1, 32, 16), (6, 2, 64, 16), (32, 8, 128, 16), (16, 1, 128, 32),
+                                           (3, 3, 96, 48), (8, 2, 256, 16)])
+@pytest.mark.parametrize("nsplit", [1, 3, 16])
+def test_decode_attention_on_the_matrix_cores(ops, nh, nkv, d, page, nsplit):
+    """Single tokens of several requests at once, against the plain attention, with the
+    key range cut into parts; lengths chosen at block and page edges."""
+    dtype = torch.bfloat16
+    assert ops.decode_attention_supported(nh, nkv, d, page, dtype)
+    seq_lens = [1, 15, 16, 17, 95, 96, 97, 300, 641]
+    R = len(seq_lens)
+    kc, vc, table, dense = paged_setup(seq_lens, nkv, d, page, dtype, seed=d + nsplit)
+    q = rnd(R + 1, nh * d, dtype=dtype, seed=2)  # one padding token at the end
+    positions = torch.tensor([n - 1 for n in seq_lens] + [0], dtype=torch.int32, device=DEV)
+    token_req = torch.tensor(list(range(R)) + [-1], dtype=torch.int32, device=DEV)
+    slots = torch.arange(1, R + 1, dtype=torch.int32, device=DEV)
+    out = torch.full((R + 1, nh * d), float("nan"), dtype=dtype, device=DEV)
+    part_o = torch.full(((R + 1) * nh * nsplit, d), float("nan"), device=DEV)
+    part_ml = torch.full(((R + 1) * nh * nsplit, 2), float("nan"), device=DEV)
+    scale = d ** -0.5
+    ops.decode_attention(out, q, kc, vc, table=table, positions=positions, token_req=token_req,
+                         slots=slots, nh=nh, nkv=nkv, d=d, scale=scale, nsplit=nsplit,
+                         part_o=part_o, part_ml=part_ml)
+    got = out.double().cpu().view(R + 1, nh, d)
+    assert torch.all(got[R] == 0)
+    qd = q.double().cpu().view(R + 1, nh, d)
+    for r, n in enumerate(seq_lens):
+        k, v = dense[r][0].double(), dense[r][1].double()
+        full_q = torch.zeros(n, nh, d, dtype=torch.float64)
+        full_q[n - 1] = qd[r]
+        want = plain.causal_gqa_attention(full_q, k, v, scale)[n - 1]
+        assert torch.allclose(got[r], want, atol=1e-2, rtol=1e-2), f"length {n}"
+    # the general kernel gives the same answer
+    ref = torch.empty_like(out)
+    ops.paged_attention(ref, q, kc, vc, table=table, positions=positions, token_req=token_req,
+                        slots=slots, nh=nh, nkv=nkv, d=d, scale=scale)
+    assert torch.allclose(out.float(), ref.float(), atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("nsplit", [1, 5])
+def test_decode_attention_far_key_and_window(ops, nsplit):
+    dtype = torch.bfloat16
+    nh, nkv, d, page, n = 8, 2, 64, 16, 700
+    part_o = torch.empty(nh * nsplit, d, device=DEV)
+    part_ml = torch.empty(nh * nsplit, 2, device=DEV)
+    args = dict(positions=torch.tensor([n - 1], dtype=torch.int32, device=DEV),
+                token_req=torch.zeros(1, dtype=torch.int32, device=DEV),
+                slots=torch.ones(1, dtype=torch.int32, device=DEV), nh=nh, nkv=nkv, d=d,
+                scale=d ** -0.5, nsplit=nsplit, part_o=part_o, part_ml=part_ml)
+    for special in [0, 15, 16, 351, 639, 640, 698, 699]:
+        kc, vc, table, dense = paged_setup([n], nkv, d, page, dtype, seed=special)
+        q = rnd(1, nh * d, dtype=dtype, seed=3)
+        qd = q.float().view(nh, d)
+        key = qd[:4].mean(0)  # matches the four heads of kv head 0
+        key = key * (60.0 / float((qd[0] * key).sum() * d ** -0.5))
+        pg, off = int(table[1, special // page]), special % page
+        kc[pg, 0, off] = key.to(dtype)
+        out = torch.empty(1, nh * d, dtype=dtype, device=DEV)
+        ops.decode_attention(out, q, kc, vc, table=table, **args)
+        assert torch.allclose(out.float().cpu().view(nh, d)[0], vc[pg, 0, :, off].float().cpu(), atol=3e-2), special
+    # window: only the last w keys count; pages behind it may be the null page
+    w = 40
+    kc, vc, table, dense = paged_setup([n], nkv, d, page, dtype, seed=77)
+    q = rnd(1, nh * d, dtype=dtype, seed=4)
+    out = torch.empty(1, nh * d, dtype=dtype, device=DEV)
+    table2 = table.clone()
+    table2[1, : (n - w) // page] = 0
+    ops.decode_attention(out, q, kc, vc, table=table2, window=w, **args)
+    k, v = dense[0][0].double(), dense[0][1].double()
+    full_q = torch.zeros(n, nh, d, dtype=torch.float64)
+    full_q[n - 1] = q.double().cpu().view(nh, d)
+    want = plain.causal_gqa_attention(full_q, k, v, d ** -0.5, window=w)[n - 1]
+    assert torch.allclose(out.double().cpu().view(nh, d), want, atol=1e-2, rtol=1e-2)
+
+
+def test_decode_attention_says_what_it_does_not_serve(ops):
+    assert not ops.decode_attention_supported(4, 2, 48, 16, torch.bfloat16)   # head size not x32
+    assert not ops.decode_attention_supported(4, 2, 64, 8, torch.bfloat16)    # page not x16
+    assert not ops.decode_attention_supported(34, 2, 64, 16, torch.bfloat16)  # 17 heads a group
+    assert not ops.decode_attention_supported(4, 2, 64, 16, torch.float32)
 
 
 def test_paged_attention_refuses_unsupported_head_sizes(ops):
