@@ -89,10 +89,112 @@ __global__ void add_rmsnorm_kernel(T* __restrict__ out, float* __restrict__ resi
   for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = from_float<T>(weight[i] * (r[i] * inv));
 }
 
+// Fast path for rows whose width is a multiple of 8: a thread keeps its 8-element chunks
+// in registers, so residual and delta are read once, with 16- and 32-byte accesses that
+// are all in flight together.  The order of the additions in the sum of squares is
+// fixed by the width alone.
+__device__ __forceinline__ void load8(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float* v) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ void store8(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float* v) {
+  uint4 a;
+  a.x = f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16);
+  a.y = f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16);
+  a.z = f32_to_bf16_bits(v[4]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[5])) << 16);
+  a.w = f32_to_bf16_bits(v[6]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[7])) << 16);
+  *reinterpret_cast<uint4*>(p) = a;
+}
+
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(T* __restrict__ out,
+                                                              float* __restrict__ residual,
+                                                              const T* __restrict__ delta,
+                                                              const float* __restrict__ weight,
+                                                              float eps, int H) {
+  __shared__ float scratch[16];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * H;
+  float v[NCH][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int e = (c * 256 + threadIdx.x) * 8;
+    if (e < H) {
+      load8(residual + base + e, v[c]);
+      if (delta != nullptr) {
+        float d[8];
+        load8(delta + base + e, d);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[c][i] += d[i];
+        store8(residual + base + e, v[c]);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += v[c][i] * v[c][i];
+    }
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = rsqrtf(total / static_cast<float>(H) + eps);
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int e = (c * 256 + threadIdx.x) * 8;
+    if (e < H) {
+      float w[8], y[8];
+      load8(weight + e, w);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = w[i] * (v[c][i] * inv);
+      store8(out + base + e, y);
+    }
+  }
+}
+
+template <typename T>
+static bool launch_add_rmsnorm_vec(T* out, float* residual, const T* delta, const float* weight,
+                                   float eps, int rows, int H, hipStream_t stream) {
+  const auto misaligned = [](const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) != 0; };
+  if (H % 8 || H > 8 * 2048 || misaligned(out, 16) || misaligned(residual, 16) ||
+      misaligned(weight, 16) || (delta != nullptr && misaligned(delta, 16)))
+    return false;
+  const int nch = (H + 2047) / 2048;
+#define KVC_NORM_CASE(NN)                                                                        \
+  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, NN>), dim3(rows), dim3(256), 0, stream, out,     \
+                     residual, delta, weight, eps, H)
+  if (nch <= 1) KVC_NORM_CASE(1);
+  else if (nch <= 2) KVC_NORM_CASE(2);
+  else if (nch <= 4) KVC_NORM_CASE(4);
+  else KVC_NORM_CASE(8);
+#undef KVC_NORM_CASE
+  return true;
+}
+
 extern "C" int kvc_add_rmsnorm(void* out, float* residual, const void* delta, const float* weight,
                                float eps, int T, int H, int dtype, kvc_stream stream) {
   if (T < 0 || H <= 0) return kvc_fail("kvc_add_rmsnorm: bad sizes");
   if (T == 0) return 0;
+  {
+    bool done = false;
+    if (dtype == 0)
+      done = launch_add_rmsnorm_vec(static_cast<float*>(out), residual,
+                                    static_cast<const float*>(delta), weight, eps, T, H, S(stream));
+    else if (dtype == 1)
+      done = launch_add_rmsnorm_vec(static_cast<bf16_t*>(out), residual,
+                                    static_cast<const bf16_t*>(delta), weight, eps, T, H, S(stream));
+    if (done) return kvc_check_launch("kvc_add_rmsnorm");
+  }
   KVC_DISPATCH_DTYPE(dtype, Tp,
                      hipLaunchKernelGGL(add_rmsnorm_kernel<Tp>, dim3(T), dim3(256), 0, S(stream),
                                         static_cast<Tp*>(out), residual,
@@ -163,11 +265,37 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gate_
   out[idx] = from_float<T>(s * u);
 }
 
+template <typename T>
+__global__ void silu_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ gate_up, int I8,
+                                    int64_t n8) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n8) return;
+  const int64_t t = idx / I8;
+  const int64_t i = (idx - t * I8) * 8;
+  const int64_t I = static_cast<int64_t>(I8) * 8;
+  float g[8], u[8], y[8];
+  load8(gate_up + t * 2 * I + i, g);
+  load8(gate_up + t * 2 * I + I + i, u);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) y[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+  store8(out + t * I + i, y);
+}
+
 extern "C" int kvc_silu_mul(void* out, const void* gate_up, int T, int I, int dtype,
                             kvc_stream stream) {
   if (T < 0 || I <= 0) return kvc_fail("kvc_silu_mul: bad sizes");
   const int64_t n = static_cast<int64_t>(T) * I;
   if (n == 0) return 0;
+  if (I % 8 == 0 && (reinterpret_cast<uintptr_t>(out) % 16) == 0 &&
+      (reinterpret_cast<uintptr_t>(gate_up) % 16) == 0) {
+    const int64_t n8 = n / 8;
+    const unsigned vblocks = static_cast<unsigned>((n8 + 255) / 256);
+    KVC_DISPATCH_DTYPE(dtype, Tp,
+                       hipLaunchKernelGGL(silu_mul_vec_kernel<Tp>, dim3(vblocks), dim3(256), 0,
+                                          S(stream), static_cast<Tp*>(out),
+                                          static_cast<const Tp*>(gate_up), I / 8, n8));
+    return kvc_check_launch("kvc_silu_mul");
+  }
   const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
   KVC_DISPATCH_DTYPE(dtype, Tp,
                      hipLaunchKernelGGL(silu_mul_kernel<Tp>, dim3(blocks), dim3(256), 0, S(stream),

@@ -1,0 +1,239 @@
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for few rows (M <= 64), bfloat16 operands,
+// float32 sums: the decode-time shape, where the weight matrix is read once from HBM
+// and everything else is small.
+//
+// The weight rows are the A operand of v_mfma_f32_16x16x32_bf16 and the activations
+// its B operand, so a lane loads 16 bytes of one weight row per instruction and a
+// wave walks 16 rows along K:
+//
+//   C^T[16 weight rows, 16 tokens] += W[16 rows, 32 k] * A^T[32 k, 16 tokens]
+//
+// A block owns 16 weight rows; its waves split K and their partial tiles are added in
+// wave order through LDS, so every element is summed in an order that K and the launch
+// shape fix, whatever M is and whatever else is in the batch.  With N/16 blocks times
+// KS waves there are enough 16-byte loads in flight to keep HBM busy.
+
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+
+#include "device_utils.h"
+#include "kvcore_hip.h"
+
+using namespace kvc;
+
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8_t zero8() {
+  bf16x8_t z;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) z[e] = static_cast<__bf16>(0.f);
+  return z;
+}
+
+template <typename OutT>
+__device__ __forceinline__ void store4(OutT* p, f32x4_t v, int n_left);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, f32x4_t v, int n_left) {
+  if (n_left >= 4 && (reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+    *reinterpret_cast<f32x4_t*>(p) = v;
+  } else {
+    for (int i = 0; i < 4 && i < n_left; ++i) p[i] = v[i];
+  }
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v, int n_left) {
+  if (n_left >= 4 && (reinterpret_cast<uintptr_t>(p) & 7) == 0) {
+    uint2 packed;
+    packed.x = f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16);
+    packed.y = f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16);
+    *reinterpret_cast<uint2*>(p) = packed;
+  } else {
+    for (int i = 0; i < 4 && i < n_left; ++i) p[i].bits = f32_to_bf16_bits(v[i]);
+  }
+}
+
+template <int RT, int NT, typename OutT>
+__global__ void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restrict__ A,
+                                   const bf16_t* __restrict__ W, const bf16_t* __restrict__ bias,
+                                   int M, int N, int K, int64_t lda, int64_t ldc, int k_per_wave) {
+  extern __shared__ float red[];  // [waves - 1][RT * NT][64][4]
+  const int wave = threadIdx.x >> 6;
+  const int waves = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 15;
+  const int quad = lane >> 4;
+  const int n0 = blockIdx.x * (16 * RT);
+  const int k_begin = wave * k_per_wave;
+  const int k_end = (k_begin + k_per_wave < K) ? k_begin + k_per_wave : K;
+
+  const bf16_t* wp[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int r = n0 + rt * 16 + col;
+    wp[rt] = W + static_cast<int64_t>(r < N ? r : N - 1) * K + 8 * quad;
+  }
+  const bf16_t* ap[NT];
+  bool tok_ok[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int tok = nt * 16 + col;
+    tok_ok[nt] = tok < M;
+    ap[nt] = A + static_cast<int64_t>(tok_ok[nt] ? tok : 0) * lda + 8 * quad;
+  }
+  f32x4_t acc[RT][NT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  // whole 32-wide steps first (no predicates, so the loads of several steps overlap), then
+  // one guarded step for a tail that is a multiple of 8
+  const int k_full = k_begin + ((k_end - k_begin) / 32) * 32;
+#pragma unroll 2
+  for (int k = k_begin; k < k_full; k += 32) {
+    bf16x8_t a[RT], b[NT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) a[rt] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) b[nt] = *reinterpret_cast<const bf16x8_t*>(ap[nt] + k);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt], b[nt], acc[rt][nt], 0, 0, 0);
+  }
+  if (k_full < k_end) {
+    const bool valid = k_full + 8 * quad < k_end;
+    bf16x8_t a[RT], b[NT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+      a[rt] = valid ? *reinterpret_cast<const bf16x8_t*>(wp[rt] + k_full) : zero8();
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      b[nt] = valid ? *reinterpret_cast<const bf16x8_t*>(ap[nt] + k_full) : zero8();
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt], b[nt], acc[rt][nt], 0, 0, 0);
+  }
+
+  constexpr int TILES = RT * NT;
+  if (wave > 0) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        *reinterpret_cast<f32x4_t*>(
+            red + ((static_cast<int64_t>(wave - 1) * TILES + rt * NT + nt) * 64 + lane) * 4) = acc[rt][nt];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  for (int w = 1; w < waves; ++w) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        acc[rt][nt] += *reinterpret_cast<const f32x4_t*>(
+            red + ((static_cast<int64_t>(w - 1) * TILES + rt * NT + nt) * 64 + lane) * 4);
+  }
+  // acc[rt][nt][i] = C[token nt*16 + col][n0 + rt*16 + 4*quad + i]; columns of unused tokens
+  // multiplied whatever row 0 of A holds and are dropped here
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int n_first = n0 + rt * 16 + 4 * quad;
+    const int n_left = N - n_first;
+    if (n_left <= 0) continue;
+    f32x4_t bv = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (bias != nullptr)
+      for (int i = 0; i < 4 && i < n_left; ++i) bv[i] = to_float(bias[n_first + i]);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int tok = nt * 16 + col;
+      if (tok >= M) continue;
+      store4<OutT>(C + static_cast<int64_t>(tok) * ldc + n_first, acc[rt][nt] + bv, n_left);
+    }
+  }
+}
+
+template <int RT, int NT, typename OutT>
+void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
+            int64_t lda, int64_t ldc, int waves, int k_per_wave, hipStream_t stream) {
+  const size_t lds = static_cast<size_t>(waves - 1) * RT * NT * 64 * 4 * sizeof(float);
+  hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, OutT>), dim3((N + 16 * RT - 1) / (16 * RT)),
+                     dim3(waves * 64), lds, stream, C, A, W, bias, M, N, K, lda, ldc, k_per_wave);
+}
+
+// The launch shape is a function of N and K alone, so that a row's sums do not depend on
+// how many rows come with it.  KVC_SKINNY_RT / KVC_SKINNY_WAVES override it for tuning.
+inline void pick_shape(int N, int K, int* rt_out, int* waves_out) {
+  // measured on MI355X at M = 1 and 8: wide outputs want 64 rows a block and 4 waves along
+  // K, narrow ones 16 rows and as many waves as K allows
+  int rt = 1, waves = 1;
+  if (N >= 16384) {
+    rt = 4;
+    waves = 4;
+  } else {
+    while (waves < 16 && K / (waves * 2) >= 128) waves *= 2;
+  }
+  if (const char* e = getenv("KVC_SKINNY_RT")) rt = atoi(e);
+  if (const char* e = getenv("KVC_SKINNY_WAVES")) waves = atoi(e);
+  *rt_out = rt;
+  *waves_out = waves;
+}
+
+template <typename OutT>
+int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
+             int64_t lda, int64_t ldc, hipStream_t stream) {
+  int rt, waves;
+  pick_shape(N, K, &rt, &waves);
+  const int nt = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
+  if ((waves - 1) * rt * nt * 1024 > 65536) return kvc_fail("kvc_gemm_skinny_bf16: launch shape needs too much LDS");
+  int k_per_wave = (K + waves - 1) / waves;
+  k_per_wave = (k_per_wave + 31) / 32 * 32;
+#define KVC_SKINNY(RT_, NT_) \
+  launch<RT_, NT_, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream)
+  const int key = rt * 10 + nt;
+  switch (key) {
+    case 11: KVC_SKINNY(1, 1); break;
+    case 12: KVC_SKINNY(1, 2); break;
+    case 14: KVC_SKINNY(1, 4); break;
+    case 21: KVC_SKINNY(2, 1); break;
+    case 22: KVC_SKINNY(2, 2); break;
+    case 24: KVC_SKINNY(2, 4); break;
+    case 41: KVC_SKINNY(4, 1); break;
+    case 42: KVC_SKINNY(4, 2); break;
+    case 44: KVC_SKINNY(4, 4); break;
+    default: return kvc_fail("kvc_gemm_skinny_bf16: unsupported launch shape");
+  }
+#undef KVC_SKINNY
+  return kvc_check_launch("kvc_gemm_skinny_bf16");
+}
+
+}  // namespace
+
+extern "C" int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M,
+                                    int N, int K, int64_t lda, int64_t ldc, int out_dtype,
+                                    kvc_stream stream) {
+  if (M < 0 || M > 64 || N <= 0 || K <= 0 || lda < K || ldc < N)
+    return kvc_fail("kvc_gemm_skinny_bf16: bad sizes (1 to 64 rows)");
+  if (K % 8 || lda % 8)
+    return kvc_fail("kvc_gemm_skinny_bf16: K and the row stride must be multiples of 8");
+  if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15))
+    return kvc_fail("kvc_gemm_skinny_bf16: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (out_dtype == 0)
+    return dispatch<float>(static_cast<float*>(C), static_cast<const bf16_t*>(A),
+                           static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N,
+                           K, lda, ldc, s);
+  if (out_dtype == 1)
+    return dispatch<bf16_t>(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
+                            static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N,
+                            K, lda, ldc, s);
+  return kvc_fail("kvc_gemm_skinny_bf16: unknown output dtype code");
+}

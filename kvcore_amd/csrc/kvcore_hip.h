@@ -86,6 +86,12 @@ int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* q, 
 int kvc_gemm_f32(float* C, const float* A, const float* W, const float* bias, int M, int N,
                  int K, int64_t lda, int64_t ldc, kvc_stream stream);
 
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) for M <= 64 rows of bfloat16 on the matrix
+// cores, float32 sums, weights streamed once; C is float32 (out_dtype 0) or bfloat16 (1).
+// K and lda must be multiples of 8, A and W 16-byte aligned.
+int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
+                         int K, int64_t lda, int64_t ldc, int out_dtype, kvc_stream stream);
+
 // table[triples[3i], triples[3i+1]] = triples[3i+2] for i < n.
 int kvc_table_update(int32_t* table, int table_stride, int table_rows, const int32_t* triples,
                      int n, kvc_stream stream);

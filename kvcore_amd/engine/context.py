@@ -56,28 +56,31 @@ class CacheGroupView:
 
 class StepBuffers:
     """Named device buffers that live across steps, so a step allocates nothing once
-    the largest batch has been seen.  ``get`` returns a view of the first ``rows`` rows."""
+    the largest batch has been seen.  ``get`` returns a view of the first ``rows`` rows.
 
-    def __init__(self, device: torch.device) -> None:
+    Buffers indexed by token are allocated for ``token_capacity`` rows at once.  A buffer
+    that still has to grow is replaced by a new tensor; ``on_grow`` is then called first,
+    because a captured graph holds the old address."""
+
+    def __init__(self, device: torch.device, token_capacity: int = 0, on_grow=None) -> None:
         self.device = device
+        self.token_capacity = token_capacity
+        self.on_grow = on_grow
         self._store: dict[str, torch.Tensor] = {}
         self.frozen = False
 
-    def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
+    def get(self, name: str, rows: int, cols: int, dtype: torch.dtype, reserve: int = 0) -> torch.Tensor:
         buf = self._store.get(name)
         if buf is None or buf.dtype != dtype or buf.shape[1] != cols or buf.shape[0] < rows:
             if self.frozen:
                 raise RuntimeError(
-                    f"step buffer {name!r} would have to grow to {rows}x{cols} while buffers are "
-                    "frozen (a captured graph holds their addresses)"
-                )
-            cap = max(rows, 1 if buf is None or buf.shape[1] != cols or buf.dtype != dtype else buf.shape[0])
-            buf = torch.empty((cap, cols), dtype=dtype, device=self.device)
+                    f"step buffer {name!r} would have to grow to {rows}x{cols} while a graph is "
+                    "being captured")
+            if buf is not None and self.on_grow is not None:
+                self.on_grow()
+            buf = torch.empty((max(rows, reserve, 1), cols), dtype=dtype, device=self.device)
             self._store[name] = buf
         return buf[:rows]
-
-    def reserve(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> None:
-        self.get(name, rows, cols, dtype)
 
 
 @dataclass
@@ -112,4 +115,5 @@ class StepContext:
 
     def buf(self, name: str, cols: int, dtype: torch.dtype | None = None, rows: int | None = None) -> torch.Tensor:
         return self.buffers.get(name, self.num_tokens if rows is None else rows, cols,
-                                self.dtype if dtype is None else dtype)
+                                self.dtype if dtype is None else dtype,
+                                reserve=self.buffers.token_capacity if rows is None else 0)

@@ -95,7 +95,8 @@ class EngineCore:
         self.runner = ModelRunner(model, page_size=self.page_size, num_pages=self.num_pages,
                                   max_num_seqs=sched.max_num_seqs,
                                   max_num_tokens=sched.max_num_scheduled_tokens,
-                                  max_model_len=self.max_model_len)
+                                  max_model_len=self.max_model_len,
+                                  use_hip_graphs=config.device_config.use_hip_graphs)
         self.sampler = Sampler(device, sched.max_num_seqs, engine_seed=config.load_config.seed)
         self.tokenizer_manager = None
         if model_json:

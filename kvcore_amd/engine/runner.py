@@ -86,7 +86,8 @@ class ModelRunner:
     buffers and the model; runs steps."""
 
     def __init__(self, model: DecoderModel, *, page_size: int, num_pages: int | Sequence[int],
-                 max_num_seqs: int, max_num_tokens: int, max_model_len: int) -> None:
+                 max_num_seqs: int, max_num_tokens: int, max_model_len: int,
+                 use_hip_graphs: bool = True) -> None:
         ops.load()  # fail here, loudly, if the kernels are not there
         if model.device.type != "cuda":
             raise RuntimeError("kvcore_amd runs on a GPU only; there is no CPU path")
@@ -114,7 +115,8 @@ class ModelRunner:
             torch.zeros((max_num_seqs, *sa.need.shape), dtype=sa.need.dtype, device=self.device)
             for sa in model.state_arrays
         ]
-        self.buffers = StepBuffers(self.device)
+        self.buffers = StepBuffers(self.device, token_capacity=max_num_tokens,
+                                   on_grow=self._drop_graphs)
 
         # host mirror of what each slot's table rows hold: (request id, entries synced,
         # leading entries nulled) per group
@@ -141,6 +143,20 @@ class ModelRunner:
         self._np = {name: self._meta_np[o:o + n] for name, (o, n) in self._off.items()}
         self._copy_done = torch.cuda.Event()
         self._copy_pending = False
+
+        # steps of single tokens are captured once per batch-size bucket and replayed
+        self.use_hip_graphs = use_hip_graphs and model.graph_safe()
+        self._graph_buckets = _decode_buckets(min(max_num_seqs, max_num_tokens))
+        self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        self._graph_warm: set[int] = set()
+        self.graph_replays = 0
+
+    def _drop_graphs(self) -> None:
+        """A step buffer is about to move: captured graphs hold its old address."""
+        if getattr(self, "_graphs", None):
+            torch.cuda.synchronize(self.device)
+            self._graphs.clear()
+            self._graph_warm.clear()
 
     # -------------------------------------------------------------------- bookkeeping
     def forget(self, slot: int) -> None:
@@ -246,6 +262,20 @@ class ModelRunner:
         T = t
         npv["q_start"][R] = T
 
+        # a step of single tokens that all want their logits runs padded to a bucket size,
+        # so that one captured graph serves every batch of that bucket
+        bucket = 0
+        if self.use_hip_graphs and T == R and n_rows == R and all(w == 1 for w in q_lens):
+            bucket = next((b for b in self._graph_buckets if b >= R), 0)
+        if bucket:
+            npv["token_ids"][R:bucket] = 0
+            npv["positions"][R:bucket] = 0
+            npv["token_req"][R:bucket] = -1
+            npv["logit_rows"][:bucket] = np.arange(bucket, dtype=np.int32)
+            npv["q_start"][R:bucket + 1] = np.arange(R, bucket + 1, dtype=np.int32)
+            npv["seq_lens"][R:bucket] = 0
+            npv["slots"][R:bucket] = 0
+
         updates = self._table_updates(entries)
         upd_counts = []
         cursor = self._upd_off
@@ -264,7 +294,19 @@ class ModelRunner:
             if count:
                 ops.table_update(self.groups[g].table, self._meta_dev[off:off + 3 * count], count)
 
-        ctx = StepContext(
+        ids = [e.request_id for e in entries]
+        if bucket:
+            return StepOutput(ids, self._run_decode_bucket(bucket, R), owners, T)
+        ctx = self._context(T, R, q_lens, seq_lens, max(q_lens), max(seq_lens))
+        hidden = self.model.forward(ctx)
+        logits = None
+        if n_rows:
+            logits = self.model.compute_logits(ctx, hidden, self._dev["logit_rows"], n_rows)
+        return StepOutput(ids, logits, owners, T)
+
+    def _context(self, T: int, R: int, q_lens: list[int], seq_lens: list[int], max_q: int,
+                 max_seq: int) -> StepContext:
+        return StepContext(
             num_tokens=T, num_reqs=R,
             token_ids=self._dev["token_ids"], positions=self._dev["positions"],
             token_req=self._dev["token_req"], q_start=self._dev["q_start"],
@@ -272,13 +314,51 @@ class ModelRunner:
             groups=self.groups, states=self.states, buffers=self.buffers,
             dtype=self.dtype, device=self.device,
             host_query_lens=q_lens, host_seq_lens=seq_lens,
-            max_query_len=max(q_lens), max_seq_len=max(seq_lens),
+            max_query_len=max_q, max_seq_len=max_seq,
         )
-        hidden = self.model.forward(ctx)
-        logits = None
-        if n_rows:
-            logits = self.model.compute_logits(ctx, hidden, self._dev["logit_rows"], n_rows)
-        return StepOutput([e.request_id for e in entries], logits, owners, T)
+
+    def _run_decode_bucket(self, bucket: int, num_live: int) -> torch.Tensor:
+        """A padded step of ``bucket`` single tokens.  The first such step runs launch by
+        launch (which also sizes every step buffer); the second is captured into a HIP
+        graph; from then on the graph is replayed.  Nothing in the graph depends on the
+        batch beyond what the index arrays on the device say: the context it was captured
+        with claims the longest sequence the engine allows."""
+
+        def run() -> torch.Tensor:
+            ctx = self._context(bucket, bucket, [1] * bucket, [self.max_model_len] * bucket, 1,
+                                self.max_model_len)
+            hidden = self.model.forward(ctx)
+            return self.model.compute_logits(ctx, hidden, self._dev["logit_rows"], bucket)
+
+        if bucket in self._graphs:
+            graph, logits = self._graphs[bucket]
+            graph.replay()
+            self.graph_replays += 1
+            return logits[:num_live]
+        if bucket not in self._graph_warm:
+            self._graph_warm.add(bucket)
+            return run()[:num_live]
+        graph = torch.cuda.CUDAGraph()
+        self.buffers.frozen = True
+        try:
+            with torch.cuda.graph(graph):
+                logits = run()
+        finally:
+            self.buffers.frozen = False
+        self._graphs[bucket] = (graph, logits)
+        graph.replay()
+        self.graph_replays += 1
+        return logits[:num_live]
+
+
+def _decode_buckets(limit: int) -> list[int]:
+    """Batch sizes at which decode steps are captured: 1, 2, 4, 8, then steps of 8 up to 64,
+    then steps of 32, always ending at the engine's limit."""
+    out = [b for b in (1, 2, 4) if b < limit]
+    out += list(range(8, min(limit, 64), 8))
+    out += list(range(64, limit, 32))
+    out.append(limit)
+    return sorted(set(out))
 
 
 def describe_model(model: DecoderModel) -> str:

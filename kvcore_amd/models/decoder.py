@@ -150,6 +150,12 @@ class DecoderModel:
             return {f"{self.spec.head_prefix}.weight"}
         return set()
 
+    def graph_safe(self) -> bool:
+        """True iff every part says its forward may be captured into a HIP graph (it reads
+        nothing from the device and decides nothing on the host per step)."""
+        owned = [part for _, part in self._owned] + list(self.positions) + list(self.blocks)
+        return all(getattr(part, "graph_safe", True) for part in owned)
+
     def num_param_bytes(self) -> int:
         return sum(bp.tensor.numel() * bp.tensor.element_size() for bp in self.params.values())
 

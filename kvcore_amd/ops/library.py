@@ -42,6 +42,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "kvc_decode_attention_supported": [I, I, I, I, I],
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
+        "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, P],
         "kvc_table_update": [P, I, I, P, I, P],
         "kvc_argmax": [P, P, I, I, L, P],
         "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P],
@@ -296,9 +297,33 @@ def gemm_f32(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Te
                                M, N, K, a.stride(0), out.stride(0), _stream()), "kvc_gemm_f32")
 
 
+SKINNY_MAX_ROWS = 64
+SKINNY_PREFERRED_ROWS = 16
+
+
+def gemm_skinny_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor,
+                     bias: torch.Tensor | None = None) -> None:
+    """``out = a @ w.T (+ bias)`` for up to 64 rows of bfloat16; ``out`` is bfloat16 or
+    float32 (the sums are float32 either way)."""
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape != (N, K) or out.shape != (M, N) or a.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm_skinny_bf16: shapes do not match")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not a.is_cuda or not out.is_cuda:
+        raise KernelError("gemm_skinny_bf16: operands must be bfloat16 GPU tensors")
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.shape != (N,)):
+        raise KernelError("gemm_skinny_bf16: bias must be bfloat16 [N]")
+    _check(load().kvc_gemm_skinny_bf16(out.data_ptr(), a.data_ptr(), _dev(w, "w"),
+                                       None if bias is None else _dev(bias, "bias"), M, N, K,
+                                       a.stride(0), out.stride(0), _code(out, "out"), _stream()),
+           "kvc_gemm_skinny_bf16")
+
+
 def linear(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -> None:
-    """``out = x @ w.T (+ bias)``.  float32 runs the library's own true-float32 kernel;
-    bfloat16 runs the vendor matrix product through torch (float32 accumulation)."""
+    """``out = x @ w.T (+ bias)``.  float32 runs the library's own true-float32 kernel.
+    bfloat16 with at most 64 rows runs the weight-streaming matrix-core kernel (float32
+    ``out`` allowed); more rows run the vendor matrix product through torch.  All sum in
+    float32."""
     if x.dtype == torch.float32:
         gemm_f32(out, x, w, bias)
         return
@@ -306,6 +331,19 @@ def linear(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tens
         raise KernelError(f"linear: unsupported operands {x.dtype}/{w.dtype} on {x.device}")
     if x.shape[0] == 0:
         return
+    M, K = x.shape
+    N = w.shape[0]
+    skinny_ok = (M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0
+                 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+    # measured on MI355X: the weight-streaming kernel wins for up to 16 rows unless K or N
+    # is very large; it is also the only one that stores float32
+    if skinny_ok and (out.dtype == torch.float32
+                      or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)):
+        gemm_skinny_bf16(out, x, w, bias)
+        return
+    if out.dtype != torch.bfloat16:
+        raise KernelError("linear: float32 output of bfloat16 operands needs at most 64 rows, "
+                          "K a multiple of 8 and aligned operands")
     if bias is None:
         torch.mm(x, w.t(), out=out)
     else:

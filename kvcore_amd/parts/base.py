@@ -84,7 +84,14 @@ class Runtime:
 
 
 class Part:
-    """Base of all parts: declares parameters, receives them bound to device tensors."""
+    """Base of all parts: declares parameters, receives them bound to device tensors.
+
+    ``graph_safe``: the part's forward only launches work on the current stream with
+    arguments fixed by the batch's size, so a step may be captured into a HIP graph and
+    replayed.  A part that reads device data on the host or loops over requests in Python
+    sets it to False, and the engine then runs every step launch by launch."""
+
+    graph_safe = True
 
     def param_specs(self) -> list[ParamSpec]:
         return []

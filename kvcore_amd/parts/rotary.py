@@ -59,8 +59,8 @@ class RotaryEncoding(PositionEncoding):
 
     def prepare(self, ctx) -> None:
         half = self.rot_dim // 2
-        cos = ctx.buffers.get(f"rope_cos_{id(self)}", ctx.num_tokens, half, torch.float32)
-        sin = ctx.buffers.get(f"rope_sin_{id(self)}", ctx.num_tokens, half, torch.float32)
+        cos = ctx.buf(f"rope_cos_{id(self)}", half, torch.float32)
+        sin = ctx.buf(f"rope_sin_{id(self)}", half, torch.float32)
         ops.rope_table(cos, sin, ctx.positions, self.inv_freq)
         ctx.scratch[self._key] = RotaryTables(cos, sin, self.rot_dim, self.interleaved)
 

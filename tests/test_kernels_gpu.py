@@ -46,7 +46,7 @@ def test_embed(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H", [96, 200, 4100])
+@pytest.mark.parametrize("H", [96, 200, 4100, 4096, 12296])
 def test_add_rmsnorm(ops, dtype, H):
     T, eps = 5, 1e-5
     residual = rnd(T, H, seed=1)
@@ -117,6 +117,49 @@ def test_gemm_f32_is_true_float32_and_does_not_depend_on_the_batch(ops, M, N, K)
     ops.gemm_f32(wide_out[:, :N], wide_in[:, :K], w, None)
     assert torch.equal(wide_out[:, :N], out - b) or torch.allclose(wide_out[:, :N], out - b, atol=1e-5)
     assert torch.all(wide_out[:, N:] == 0)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 16, 64), (5, 100, 200), (8, 4096, 4096), (16, 130, 1032),
+                                   (17, 6144, 512), (33, 48, 14336), (64, 1000, 2048)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_skinny_bf16(ops, M, N, K, out_dtype):
+    a = rnd(M, K, dtype=torch.bfloat16, seed=1)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=2, scale=0.05)
+    bias = rnd(N, dtype=torch.bfloat16, seed=3)
+    out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+    ops.gemm_skinny_bf16(out, a, w, bias)
+    want = a.double() @ w.double().T + bias.double()
+    mag = a.double().abs() @ w.double().abs().T + bias.double().abs()
+    err = (out.double() - want).abs()
+    # float32 sums of exact bfloat16 products; a bfloat16 result adds one rounding of 2^-9
+    bound = 8 * math.sqrt(K) * 2 ** -24 * mag + 1e-6
+    if out_dtype == torch.bfloat16:
+        bound = bound + want.abs() * 2 ** -8
+    assert (err <= bound).all(), float((err / bound).max())
+    # a row alone, or in another place of the batch, gives the same bits
+    single = torch.empty(1, N, dtype=out_dtype, device=DEV)
+    for i in {0, M // 2, M - 1}:
+        ops.gemm_skinny_bf16(single, a[i:i + 1].contiguous(), w, bias)
+        assert torch.equal(single[0], out[i])
+    # strided rows in and out, no bias
+    wide_in = torch.zeros(M, K + 8, dtype=torch.bfloat16, device=DEV)
+    wide_in[:, :K] = a
+    wide_out = torch.zeros(M, N + 3, dtype=out_dtype, device=DEV)
+    ops.gemm_skinny_bf16(wide_out[:, :N], wide_in[:, :K], w, None)
+    ref = torch.empty(M, N, dtype=out_dtype, device=DEV)
+    ops.gemm_skinny_bf16(ref, a, w, None)
+    assert torch.equal(wide_out[:, :N], ref) and torch.all(wide_out[:, N:] == 0)
+
+
+def test_linear_picks_a_kernel_by_row_count(ops):
+    w = rnd(96, 256, dtype=torch.bfloat16, seed=5, scale=0.05)
+    for M in (3, 64, 65, 200):
+        x = rnd(M, 256, dtype=torch.bfloat16, seed=M)
+        out = torch.empty(M, 96, dtype=torch.bfloat16, device=DEV)
+        ops.linear(out, x, w)
+        assert torch.allclose(out.double(), x.double() @ w.double().T, atol=2e-2, rtol=2e-2)
+    with pytest.raises(ops.KernelError):
+        ops.linear(torch.empty(100, 96, device=DEV), rnd(100, 256, dtype=torch.bfloat16), w)
 
 
 def test_bf16_linear_uses_float32_accumulation(ops):

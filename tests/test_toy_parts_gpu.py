@@ -29,6 +29,8 @@ def register_toy():
         """y_t = W s_t with s_t = decay * s_{t-1} + x_t per request: the state s is the
         mixer's own, one row per request slot, carried across steps."""
 
+        graph_safe = False  # loops over requests on the host
+
         def __init__(self, *, hidden_size, decay, position=None):
             self.hidden_size, self.decay = hidden_size, decay
 
