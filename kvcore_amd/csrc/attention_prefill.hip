@@ -1,0 +1,336 @@
+// Paged attention for portions of prompts, bfloat16, on the matrix cores.
+//
+// A block of four waves owns up to 64*CT query rows of one request and one kv head:
+// BQ = 64*CT / g consecutive tokens times the g query heads that share the kv head.
+// It walks the request's keys in tiles of 64, staged once through LDS for all four
+// waves: K pages as they lie in the cache ([key, d], rows padded against bank
+// conflicts) and V pages as they lie there ([d, key]).  Per wave, per 16-key block:
+//
+//   S^T[16 keys, 16 rows]  = K[16 keys, d]   * Q^T[d, 16 rows]        (16x16x32, CT times)
+//   O^T[d, 16 rows]       += V^T[d, 16 keys] * P^T[16 keys, 16 rows]  (16x16x16, CT times)
+//
+// The accumulator layout of S^T is the B-operand layout of the second product, so the
+// probabilities stay in registers.  Softmax state is float32 per row; the running
+// output is rescaled once per 64-key tile and only when some row's maximum moved.
+// A key is visible to a row iff first <= key <= the row's position; keys beyond the
+// request's last position and pages given back behind a window are zeroed on their way
+// into LDS, so nothing that was not written by this request reaches a product.
+
+#include <hip/hip_runtime.h>
+
+#include "device_utils.h"
+#include "kvcore_hip.h"
+
+using namespace kvc;
+
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kWaves = 4;
+constexpr int kKeyBlocks = 4;  // 16-key blocks per LDS tile
+
+template <int D, int CT>
+__global__ __launch_bounds__(kWaves * 64) void prefill_attention_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ table, int table_stride, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int num_reqs, int nh,
+    int nkv, int page_size, int num_pages, float scale_log2e, int window) {
+  constexpr int NJ = D / 16;
+  constexpr int NC = D / 32;
+  constexpr int KROW = D + 8;  // padded K row in LDS (elements)
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[kKeyBlocks * 16 * KROW];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[kKeyBlocks * D * 16];
+
+  const int g = nh / nkv;
+  const int bq = (64 * CT) / g;  // tokens per block
+  const int hk = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int col = lane & 15;
+  const int quad = lane >> 4;
+
+  // which request and which of its token tiles: tiles are numbered request by request
+  int req = -1, t0 = 0, t_end = 0;
+  {
+    int tile = blockIdx.x;
+    for (int r = 0; r < num_reqs; ++r) {
+      const int b = q_start[r], e = q_start[r + 1];
+      const int tiles = (e - b + bq - 1) / bq;
+      if (tile < tiles) {
+        req = r;
+        t0 = b + tile * bq;
+        t_end = (t0 + bq < e) ? t0 + bq : e;
+        break;
+      }
+      tile -= tiles;
+    }
+  }
+  if (req < 0) return;  // the grid is an upper bound on the number of tiles
+  const int n_tok = t_end - t0;
+  const int32_t* row_table = table + static_cast<int64_t>(slots[req]) * table_stride;
+  const int pos_lo = positions[t0];
+  const int pos_hi = positions[t_end - 1];  // positions rise by one along a request's tokens
+  const int first_lo = (window > 0 && pos_lo - window + 1 > 0) ? pos_lo - window + 1 : 0;
+
+  // this lane's rows: column `col` of tile ct is row (wave*CT + ct)*16 + col of the block
+  int my_pos[CT], my_first[CT], my_tok[CT], my_head[CT];
+  bool live[CT];
+  bf16x8_t qb[CT][NC];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int rho = (wave * CT + ct) * 16 + col;
+    const int tq = rho / g;
+    live[ct] = tq < n_tok;
+    my_tok[ct] = t0 + (live[ct] ? tq : 0);
+    my_head[ct] = hk * g + rho % g;
+    my_pos[ct] = live[ct] ? positions[my_tok[ct]] : -1;
+    my_first[ct] = (window > 0 && my_pos[ct] - window + 1 > 0) ? my_pos[ct] - window + 1 : 0;
+    const bf16_t* qp = q + static_cast<int64_t>(my_tok[ct]) * q_stride +
+                       static_cast<int64_t>(my_head[ct]) * D + 8 * quad;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      if (live[ct]) {
+        qb[ct][c] = *reinterpret_cast<const bf16x8_t*>(qp + 32 * c);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qb[ct][c][e] = static_cast<__bf16>(0.f);
+      }
+    }
+  }
+  // wave-uniform bounds of what this wave's rows can see
+  int wave_pos_hi = -1;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) wave_pos_hi = max(wave_pos_hi, my_pos[ct]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) wave_pos_hi = max(wave_pos_hi, __shfl_xor(wave_pos_hi, o, 64));
+
+  f32x4_t o_acc[CT][NJ];
+  float m[CT], l[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    m[ct] = -INFINITY;
+    l[ct] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) o_acc[ct][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int blocks_per_page = page_size / 16;
+  const int kb_first = first_lo / 16;
+  const int kb_end = pos_hi / 16 + 1;
+  constexpr int K_CHUNKS = kKeyBlocks * 16 * (D / 8);  // 16-byte pieces of a K tile
+  constexpr int V_CHUNKS = kKeyBlocks * D * 2;         // 16-byte pieces of a V tile
+  constexpr int K_PER_THREAD = K_CHUNKS / (kWaves * 64);
+  constexpr int V_PER_THREAD = V_CHUNKS / (kWaves * 64);
+
+  for (int kb0 = kb_first; kb0 < kb_end; kb0 += kKeyBlocks) {
+    // ---- stage the tile: global -> registers -> LDS
+    uint4 kreg[K_PER_THREAD], vreg[V_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < K_PER_THREAD; ++i) {
+      const int chunk = i * (kWaves * 64) + tid;
+      const int key_row = chunk / (D / 8);  // 0 .. 63 within the tile
+      const int piece = chunk - key_row * (D / 8);
+      const int kb = kb0 + key_row / 16;
+      const int key = kb * 16 + (key_row & 15);
+      uint4 val = make_uint4(0u, 0u, 0u, 0u);
+      if (kb < kb_end && key <= pos_hi) {
+        const int page = row_table[kb / blocks_per_page];
+        if (page > 0 && page < num_pages) {
+          const bf16_t* src = k_cache + ((static_cast<int64_t>(page) * nkv + hk) * page_size + key % page_size) * D + piece * 8;
+          val = *reinterpret_cast<const uint4*>(src);
+        }
+      }
+      kreg[i] = val;
+    }
+#pragma unroll
+    for (int i = 0; i < V_PER_THREAD; ++i) {
+      const int chunk = i * (kWaves * 64) + tid;
+      const int kbi = chunk / (D * 2);  // key block within the tile
+      const int rem = chunk - kbi * (D * 2);
+      const int drow = rem >> 1;
+      const int half = rem & 1;
+      const int kb = kb0 + kbi;
+      const int key0 = kb * 16 + half * 8;
+      uint4 val = make_uint4(0u, 0u, 0u, 0u);
+      if (kb < kb_end && key0 <= pos_hi) {
+        const int page = row_table[kb / blocks_per_page];
+        if (page > 0 && page < num_pages) {
+          const bf16_t* src = v_cache + ((static_cast<int64_t>(page) * nkv + hk) * D + drow) * page_size + key0 % page_size;
+          val = *reinterpret_cast<const uint4*>(src);
+          const int n_ok = pos_hi - key0 + 1;  // keys key0 .. key0+7 beyond pos_hi are not this request's
+          if (n_ok < 8) {
+            uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (e >= n_ok) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+            val = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+        }
+      }
+      vreg[i] = val;
+    }
+    __syncthreads();  // the previous tile has been consumed
+#pragma unroll
+    for (int i = 0; i < K_PER_THREAD; ++i) {
+      const int chunk = i * (kWaves * 64) + tid;
+      const int key_row = chunk / (D / 8);
+      const int piece = chunk - key_row * (D / 8);
+      *reinterpret_cast<uint4*>(k_lds + key_row * KROW + piece * 8) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < V_PER_THREAD; ++i) {
+      const int chunk = i * (kWaves * 64) + tid;
+      *reinterpret_cast<uint4*>(v_lds + chunk * 8) = vreg[i];
+    }
+    __syncthreads();
+
+    // ---- scores of the tile for this wave's rows
+    if (kb0 * 16 > wave_pos_hi) continue;  // nothing here is visible to this wave (uniform)
+    f32x4_t s[CT][kKeyBlocks];
+#pragma unroll
+    for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
+      bf16x8_t ka[NC];
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+        ka[c] = *reinterpret_cast<const bf16x8_t*>(k_lds + (kbi * 16 + col) * KROW + 32 * c + 8 * quad);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], qb[ct][c], acc, 0, 0, 0);
+        s[ct][kbi] = acc;
+      }
+    }
+    // ---- softmax update per row over the 64 keys of the tile
+    s16x4_t pb[CT][kKeyBlocks];
+    float alpha[CT];
+    bool moved = false;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = (kb0 + kbi) * 16 + 4 * quad + i;
+          const bool ok = key >= my_first[ct] && key <= my_pos[ct];
+          const float v = ok ? s[ct][kbi][i] * scale_log2e : -INFINITY;
+          s[ct][kbi][i] = v;
+          mx = fmaxf(mx, v);
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[ct], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha[ct] = __builtin_amdgcn_exp2f(m[ct] - m_safe);
+      moved = moved || (m_new != m[ct]);
+      float ps = 0.f;
+#pragma unroll
+      for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = __builtin_amdgcn_exp2f(s[ct][kbi][i] - m_safe);
+          ps += p;
+          pb[ct][kbi][i] = static_cast<short>(f32_to_bf16_bits(p));
+        }
+      }
+      ps += __shfl_xor(ps, 16, 64);
+      ps += __shfl_xor(ps, 32, 64);
+      l[ct] = l[ct] * alpha[ct] + ps;
+      m[ct] = m_new;
+    }
+    if (__any(moved)) {
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) o_acc[ct][j] = o_acc[ct][j] * alpha[ct];
+    }
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
+      if ((kb0 + kbi) * 16 > wave_pos_hi) break;  // uniform: later blocks weigh nothing
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const s16x4_t va = *reinterpret_cast<const s16x4_t*>(v_lds + (kbi * D + 16 * j + col) * 16 + 4 * quad);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          o_acc[ct][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb[ct][kbi], o_acc[ct][j], 0, 0, 0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    if (!live[ct]) continue;
+    const float inv = (l[ct] > 0.f) ? 1.f / l[ct] : 0.f;
+    bf16_t* op = out + (static_cast<int64_t>(my_tok[ct]) * nh + my_head[ct]) * D + 4 * quad;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const f32x4_t v = o_acc[ct][j] * inv;
+      uint2 packed;
+      packed.x = f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16);
+      packed.y = f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16);
+      *reinterpret_cast<uint2*>(op + 16 * j) = packed;
+    }
+  }
+}
+
+template <int D>
+int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t* k_cache,
+                   const bf16_t* v_cache, const int32_t* table, int table_stride,
+                   const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
+                   int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
+                   hipStream_t stream) {
+  const int g = nh / nkv;
+  constexpr int CT = 2;
+  const int bq = (64 * CT) / g;
+  const int max_tiles = (T + bq - 1) / bq + R;  // every request may end in a ragged tile
+  hipLaunchKernelGGL((prefill_attention_kernel<D, CT>), dim3(max_tiles, nkv), dim3(kWaves * 64), 0,
+                     stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
+                     q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window);
+  return kvc_check_launch("kvc_prefill_attention");
+}
+
+}  // namespace
+
+extern "C" int kvc_prefill_attention_supported(int nh, int nkv, int d, int page_size, int dtype) {
+  if (dtype != 1) return 0;
+  if (nkv <= 0 || nh % nkv || nh / nkv > 64) return 0;
+  if (page_size % 16) return 0;
+  return d == 64 || d == 128;
+}
+
+extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
+                                     const void* k_cache, const void* v_cache,
+                                     const int32_t* table, int table_stride,
+                                     const int32_t* positions, const int32_t* q_start,
+                                     const int32_t* slots, int T, int R, int nh, int nkv, int d,
+                                     int page_size, int num_pages, float scale, int window,
+                                     kvc_stream stream) {
+  if (!kvc_prefill_attention_supported(nh, nkv, d, page_size, 1))
+    return kvc_fail("kvc_prefill_attention: unsupported shape (bfloat16, head size 64 or 128, at "
+                    "most 64 query heads per kv head, page size a multiple of 16)");
+  if (T < 0 || R <= 0 || nkv > 65535 || table_stride <= 0 || num_pages <= 0)
+    return kvc_fail("kvc_prefill_attention: bad sizes");
+  if (q_stride % 8) return kvc_fail("kvc_prefill_attention: q rows must be 16-byte aligned");
+  if (T == 0) return 0;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const bf16_t* qq = static_cast<const bf16_t*>(q);
+  const bf16_t* kc = static_cast<const bf16_t*>(k_cache);
+  const bf16_t* vc = static_cast<const bf16_t*>(v_cache);
+  if (d == 64)
+    return launch_prefill<64>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
+                              positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
+                              window, s);
+  return launch_prefill<128>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
+                             positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
+                             window, s);
+}

@@ -41,6 +41,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "kvc_decode_attention_supported": [I, I, I, I, I],
+        "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
+        "kvc_prefill_attention_supported": [I, I, I, I, I],
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
         "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, P],
         "kvc_table_update": [P, I, I, P, I, P],
@@ -269,6 +271,33 @@ def decode_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
         _dev(slots, "slots", torch.int32), T, nh, nkv, d, page_size, num_pages, float(scale),
         int(window), int(nsplit), _stream()), "kvc_decode_attention")
+
+
+def prefill_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype: torch.dtype) -> bool:
+    return bool(load().kvc_prefill_attention_supported(nh, nkv, d, page_size, DTYPE_CODE.get(dtype, -1)))
+
+
+def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      *, table: torch.Tensor, positions: torch.Tensor, q_start: torch.Tensor,
+                      slots: torch.Tensor, num_reqs: int, nh: int, nkv: int, d: int, scale: float,
+                      window: int = 0) -> None:
+    """bfloat16 attention of portions of prompts on the matrix cores (see the C header)."""
+    T = out.shape[0]
+    if out.shape != (T, nh * d) or not out.is_contiguous() or out.dtype != torch.bfloat16:
+        raise KernelError("prefill_attention: out must be contiguous bfloat16 [T, nh*d]")
+    if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or q.dtype != out.dtype:
+        raise KernelError("prefill_attention: q does not fit")
+    num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "prefill_attention")
+    if k_cache.dtype != out.dtype:
+        raise KernelError("prefill_attention: cache dtype differs from the queries'")
+    if positions.numel() < T or q_start.numel() < num_reqs + 1 or slots.numel() < num_reqs:
+        raise KernelError("prefill_attention: index arrays too short")
+    _check(load().kvc_prefill_attention(
+        out.data_ptr(), q.data_ptr(), q.stride(0), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
+        _dev(table, "table", torch.int32), table.shape[1], _dev(positions, "positions", torch.int32),
+        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), T, num_reqs,
+        nh, nkv, d, page_size, num_pages, float(scale), int(window), _stream()),
+        "kvc_prefill_attention")
 
 
 def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int, who: str) -> tuple[int, int]:

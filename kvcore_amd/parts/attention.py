@@ -105,6 +105,13 @@ class PagedAttention(Mixer):
                 part_ml = ctx.buffers.get("attn_part_ml", T * self.num_heads * nsplit, 2, torch.float32)
             ops.decode_attention(attn, qkv, k_cache, v_cache, nsplit=nsplit, part_o=part_o,
                                  part_ml=part_ml, **common)
+        elif ctx.max_query_len > 1 and ops.prefill_attention_supported(
+                self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
+            # portions of prompts (single tokens may ride along): tiles of query rows per block
+            ops.prefill_attention(attn, qkv, k_cache, v_cache, table=group.table,
+                                  positions=ctx.positions, q_start=ctx.q_start, slots=ctx.slots,
+                                  num_reqs=ctx.num_reqs, nh=self.num_heads, nkv=self.num_kv_heads,
+                                  d=self.head_dim, scale=self.scale, window=self.window)
         else:
             ops.paged_attention(attn, qkv, k_cache, v_cache, **common)
         out = ctx.buf("mixer_out", self.hidden_size)

@@ -447,7 +447,76 @@ def test_decode_attention_far_key_and_window(ops, nsplit):
     assert torch.allclose(out.double().cpu().view(nh, d), want, atol=1e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,page", [(8, 2, 64, 16), (32, 8, 128, 16), (6, 2, 128, 32), (5, 1, 64, 48),
+                                           (4, 4, 128, 16), (16, 1, 64, 16)])
+def test_prefill_attention_on_the_matrix_cores(ops, nh, nkv, d, page):
+    """Portions of prompts with and without earlier context, beside single tokens, against
+    the plain attention; lengths chosen at tile, block and page edges."""
+    dtype = torch.bfloat16
+    assert ops.prefill_attention_supported(nh, nkv, d, page, dtype)
+    seq_lens = [200, 1, 33, 130, 64, 97, 700]
+    q_lens = [200, 1, 5, 1, 64, 17, 129]
+    kc, vc, table, dense = paged_setup(seq_lens, nkv, d, page, dtype, seed=d + nh)
+    T = sum(q_lens)
+    q = rnd(T, nh * d, dtype=dtype, seed=7)
+    positions, q_start = [], [0]
+    for n, ql in zip(seq_lens, q_lens):
+        positions += list(range(n - ql, n))
+        q_start.append(q_start[-1] + ql)
+    positions = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    q_start_t = torch.tensor(q_start, dtype=torch.int32, device=DEV)
+    slots = torch.arange(1, len(seq_lens) + 1, dtype=torch.int32, device=DEV)
+    out = torch.full((T, nh * d), float("nan"), dtype=dtype, device=DEV)
+    scale = d ** -0.5
+    ops.prefill_attention(out, q, kc, vc, table=table, positions=positions, q_start=q_start_t,
+                          slots=slots, num_reqs=len(seq_lens), nh=nh, nkv=nkv, d=d, scale=scale)
+    got = out.double().cpu().view(T, nh, d)
+    qd = q.double().cpu().view(T, nh, d)
+    for r, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        k, v = dense[r][0].double(), dense[r][1].double()
+        full_q = torch.zeros(n, nh, d, dtype=torch.float64)
+        full_q[n - ql:] = qd[q_start[r]:q_start[r + 1]]
+        want = plain.causal_gqa_attention(full_q, k, v, scale)[n - ql:]
+        assert torch.allclose(got[q_start[r]:q_start[r + 1]], want, atol=1e-2, rtol=1e-2), f"request {r}"
+
+
+def test_prefill_attention_far_key_and_window(ops):
+    dtype = torch.bfloat16
+    nh, nkv, d, page, n, ql = 8, 2, 64, 16, 700, 40
+    positions = torch.arange(n - ql, n, dtype=torch.int32, device=DEV)
+    args = dict(positions=positions, q_start=torch.tensor([0, ql], dtype=torch.int32, device=DEV),
+                slots=torch.ones(1, dtype=torch.int32, device=DEV), num_reqs=1, nh=nh, nkv=nkv, d=d,
+                scale=d ** -0.5)
+    for special in [0, 15, 16, 63, 64, 351, 659, 660, 698, 699]:
+        kc, vc, table, dense = paged_setup([n], nkv, d, page, dtype, seed=special)
+        q = rnd(ql, nh * d, dtype=dtype, seed=3)
+        qd = q.float().view(ql, nh, d)
+        key = qd[-1, :4].mean(0)  # matches the last token's heads of kv head 0
+        key = key * (60.0 / float((qd[-1, 0] * key).sum() * d ** -0.5))
+        pg, off = int(table[1, special // page]), special % page
+        kc[pg, 0, off] = key.to(dtype)
+        out = torch.empty(ql, nh * d, dtype=dtype, device=DEV)
+        ops.prefill_attention(out, q, kc, vc, table=table, **args)
+        assert torch.allclose(out.float().cpu().view(ql, nh, d)[-1, 0], vc[pg, 0, :, off].float().cpu(),
+                              atol=3e-2), special
+    w = 50
+    kc, vc, table, dense = paged_setup([n], nkv, d, page, dtype, seed=78)
+    q = rnd(ql, nh * d, dtype=dtype, seed=4)
+    table2 = table.clone()
+    table2[1, : (n - ql - w + 1) // page] = 0  # pages wholly behind the first row's window are gone
+    out = torch.empty(ql, nh * d, dtype=dtype, device=DEV)
+    ops.prefill_attention(out, q, kc, vc, table=table2, window=w, **args)
+    k, v = dense[0][0].double(), dense[0][1].double()
+    full_q = torch.zeros(n, nh, d, dtype=torch.float64)
+    full_q[n - ql:] = q.double().cpu().view(ql, nh, d)
+    want = plain.causal_gqa_attention(full_q, k, v, d ** -0.5, window=w)[n - ql:]
+    assert torch.allclose(out.double().cpu().view(ql, nh, d), want, atol=1e-2, rtol=1e-2)
+
+
 def test_decode_attention_says_what_it_does_not_serve(ops):
+    assert not ops.prefill_attention_supported(4, 2, 96, 16, torch.bfloat16)
+    assert not ops.prefill_attention_supported(4, 2, 64, 8, torch.bfloat16)
+    assert not ops.prefill_attention_supported(4, 2, 64, 16, torch.float32)
     assert not ops.decode_attention_supported(4, 2, 48, 16, torch.bfloat16)   # head size not x32
     assert not ops.decode_attention_supported(4, 2, 64, 8, torch.bfloat16)    # page not x16
     assert not ops.decode_attention_supported(34, 2, 64, 16, torch.bfloat16)  # 17 heads a group
