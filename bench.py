@@ -48,6 +48,8 @@ def parse_args():
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
     p.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     p.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    p.add_argument("--only-prefill", action="store_true",
+                   help="run only the 2,048-token prefill (for profiling); prints its own line")
     return p.parse_args()
 
 
@@ -158,6 +160,12 @@ def main() -> int:
             drain()
         return sorted(times[1:])[1]  # median of the three after the warm-up run
 
+    if args.only_prefill:
+        sec = prefill_run()
+        print(json.dumps({"prefill_tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3),
+                          "tokens_per_s": round(PREFILL_TOKENS / sec, 1),
+                          "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / sec / PEAK_FLOPS[args.dtype], 4)}))
+        return 0
     value, sec_per_step, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
     bytes_step = weight_bytes_per_step(cfg, esize) + kv_bytes(cfg, args.batch, mean_ctx, esize)
     achieved = bytes_step / sec_per_step

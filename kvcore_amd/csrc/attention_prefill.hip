@@ -4,14 +4,14 @@
 // BQ = 64*CT / g consecutive tokens times the g query heads that share the kv head.
 // It walks the request's keys in tiles of 64, staged once through LDS for all four
 // waves: K pages as they lie in the cache ([key, d], rows padded against bank
-// conflicts) and V pages as they lie there ([d, key]).  Per wave, per 16-key block:
+// conflicts) and V pages ([d, key]) regrouped so that operand reads are contiguous.  Per wave, per 16-key block:
 //
 //   S^T[16 keys, 16 rows]  = K[16 keys, d]   * Q^T[d, 16 rows]        (16x16x32, CT times)
 //   O^T[d, 16 rows]       += V^T[d, 16 keys] * P^T[16 keys, 16 rows]  (16x16x16, CT times)
 //
 // The accumulator layout of S^T is the B-operand layout of the second product, so the
 // probabilities stay in registers.  Softmax state is float32 per row; the running
-// output is rescaled once per 64-key tile and only when some row's maximum moved.
+// output is rescaled only when a row's maximum moved by more than 2^8.
 // A key is visible to a row iff first <= key <= the row's position; keys beyond the
 // request's last position and pages given back behind a window are zeroed on their way
 // into LDS, so nothing that was not written by this request reaches a product.
@@ -30,11 +30,21 @@ typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr float kLog2e = 1.4426950408889634f;
+
+// four float32 to four bfloat16 (round to nearest even) with the hardware's packed convert
+__device__ __forceinline__ s16x4_t pack_bf16x4(const float* p) {
+  typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+  bf16x4_t v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = static_cast<__bf16>(p[i]);
+  return *reinterpret_cast<s16x4_t*>(&v);
+}
+
 constexpr int kWaves = 4;
 constexpr int kKeyBlocks = 4;  // 16-key blocks per LDS tile
 
 template <int D, int CT>
-__global__ __launch_bounds__(kWaves * 64) void prefill_attention_kernel(
+__global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ table, int table_stride, const int32_t* __restrict__ positions,
@@ -58,7 +68,8 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_attention_kernel(
   // which request and which of its token tiles: tiles are numbered request by request
   int req = -1, t0 = 0, t_end = 0;
   {
-    int tile = blockIdx.x;
+    // late tiles of a request have the most keys: hand them out first (reverse numbering)
+    int tile = gridDim.x - 1 - blockIdx.x;
     for (int r = 0; r < num_reqs; ++r) {
       const int b = q_start[r], e = q_start[r + 1];
       const int tiles = (e - b + bq - 1) / bq;
@@ -120,6 +131,21 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_attention_kernel(
     for (int j = 0; j < NJ; ++j) o_acc[ct][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
+  // wave-uniform bounds of the positions of this wave's live rows
+  int wave_pos_lo = 0x7fffffff, wave_first_hi = 0;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    if (live[ct]) {
+      wave_pos_lo = min(wave_pos_lo, my_pos[ct]);
+      wave_first_hi = max(wave_first_hi, my_first[ct]);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    wave_pos_lo = min(wave_pos_lo, __shfl_xor(wave_pos_lo, o, 64));
+    wave_first_hi = max(wave_first_hi, __shfl_xor(wave_first_hi, o, 64));
+  }
+
   const int blocks_per_page = page_size / 16;
   const int kb_first = first_lo / 16;
   const int kb_end = pos_hi / 16 + 1;
@@ -127,42 +153,71 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_attention_kernel(
   constexpr int V_CHUNKS = kKeyBlocks * D * 2;         // 16-byte pieces of a V tile
   constexpr int K_PER_THREAD = K_CHUNKS / (kWaves * 64);
   constexpr int V_PER_THREAD = V_CHUNKS / (kWaves * 64);
+  uint4 kreg[K_PER_THREAD], vreg[V_PER_THREAD];
 
-  for (int kb0 = kb_first; kb0 < kb_end; kb0 += kKeyBlocks) {
-    // ---- stage the tile: global -> registers -> LDS
-    uint4 kreg[K_PER_THREAD], vreg[V_PER_THREAD];
+  // Fetch the tile that starts at key block kb0 into registers.  Keys beyond the request's
+  // last position, key blocks beyond the range and pages that are gone arrive as zeros.
+  // A thread's pieces of step i all lie in key block i (head size 128) or in key blocks
+  // 2i and 2i+1 (head size 64), so the page lookups are uniform or nearly so.
+  constexpr int PIECES = D / 8;               // 16-byte pieces of a K row
+  constexpr int ROWS_PER_STEP = 256 / PIECES;  // K rows that the block fetches per step
+  const int k_row0 = tid / PIECES;             // this thread's K row within a step
+  const int k_piece = tid % PIECES;
+  auto fetch_tile = [&](int kb0) {
+    const bool tail = (kb0 + kKeyBlocks) * 16 > pos_hi + 1;  // uniform: some keys are not the request's
+    int64_t kpage[kKeyBlocks], vpage[kKeyBlocks];  // element offsets of the key blocks, or -1
 #pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i) {
-      const int chunk = i * (kWaves * 64) + tid;
-      const int key_row = chunk / (D / 8);  // 0 .. 63 within the tile
-      const int piece = chunk - key_row * (D / 8);
-      const int kb = kb0 + key_row / 16;
-      const int key = kb * 16 + (key_row & 15);
-      uint4 val = make_uint4(0u, 0u, 0u, 0u);
-      if (kb < kb_end && key <= pos_hi) {
+    for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
+      const int kb = kb0 + kbi;
+      kpage[kbi] = vpage[kbi] = -1;
+      if (kb < kb_end) {
         const int page = row_table[kb / blocks_per_page];
         if (page > 0 && page < num_pages) {
-          const bf16_t* src = k_cache + ((static_cast<int64_t>(page) * nkv + hk) * page_size + key % page_size) * D + piece * 8;
-          val = *reinterpret_cast<const uint4*>(src);
+          const int sub = kb % blocks_per_page;
+          kpage[kbi] = ((static_cast<int64_t>(page) * nkv + hk) * page_size + sub * 16) * D;
+          vpage[kbi] = (static_cast<int64_t>(page) * nkv + hk) * D * page_size + sub * 16;
         }
       }
+    }
+#pragma unroll
+    for (int i = 0; i < K_PER_THREAD; ++i) {
+      const int key_row = i * ROWS_PER_STEP + k_row0;  // 0 .. 63 within the tile
+      int64_t base;
+      if constexpr (ROWS_PER_STEP == 16) {
+        base = kpage[i];
+      } else {
+        static_assert(ROWS_PER_STEP == 32, "head size 64 or 128");
+        base = (k_row0 < 16) ? kpage[2 * i] : kpage[2 * i + 1];
+      }
+      uint4 val = make_uint4(0u, 0u, 0u, 0u);
+      if (base >= 0 && (!tail || kb0 * 16 + key_row <= pos_hi))
+        val = *reinterpret_cast<const uint4*>(k_cache + base + (key_row & 15) * D + k_piece * 8);
       kreg[i] = val;
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
-      const int chunk = i * (kWaves * 64) + tid;
-      const int kbi = chunk / (D * 2);  // key block within the tile
-      const int rem = chunk - kbi * (D * 2);
+      // piece (i*256 + tid) of the tile: key block, then row of the head, then half of 16 keys
+      int kbi, rem;
+      if constexpr (D == 128) {
+        kbi = i;
+        rem = tid;
+      } else {
+        kbi = 2 * i + (tid >> 7);
+        rem = tid & 127;
+      }
       const int drow = rem >> 1;
       const int half = rem & 1;
-      const int kb = kb0 + kbi;
-      const int key0 = kb * 16 + half * 8;
+      int64_t base;
+      if constexpr (D == 128) {
+        base = vpage[i];
+      } else {
+        base = (tid < 128) ? vpage[2 * i] : vpage[2 * i + 1];
+      }
       uint4 val = make_uint4(0u, 0u, 0u, 0u);
-      if (kb < kb_end && key0 <= pos_hi) {
-        const int page = row_table[kb / blocks_per_page];
-        if (page > 0 && page < num_pages) {
-          const bf16_t* src = v_cache + ((static_cast<int64_t>(page) * nkv + hk) * D + drow) * page_size + key0 % page_size;
-          val = *reinterpret_cast<const uint4*>(src);
+      const int key0 = (kb0 + kbi) * 16 + half * 8;
+      if (base >= 0 && (!tail || key0 <= pos_hi)) {
+        val = *reinterpret_cast<const uint4*>(v_cache + base + static_cast<int64_t>(drow) * page_size + half * 8);
+        if (tail) {
           const int n_ok = pos_hi - key0 + 1;  // keys key0 .. key0+7 beyond pos_hi are not this request's
           if (n_ok < 8) {
             uint32_t w[4] = {val.x, val.y, val.z, val.w};
@@ -175,20 +230,34 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_attention_kernel(
       }
       vreg[i] = val;
     }
+  };
+
+  fetch_tile(kb_first);
+  for (int kb0 = kb_first; kb0 < kb_end; kb0 += kKeyBlocks) {
     __syncthreads();  // the previous tile has been consumed
 #pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i) {
-      const int chunk = i * (kWaves * 64) + tid;
-      const int key_row = chunk / (D / 8);
-      const int piece = chunk - key_row * (D / 8);
-      *reinterpret_cast<uint4*>(k_lds + key_row * KROW + piece * 8) = kreg[i];
-    }
+    for (int i = 0; i < K_PER_THREAD; ++i)
+      *reinterpret_cast<uint4*>(k_lds + (i * ROWS_PER_STEP + k_row0) * KROW + k_piece * 8) = kreg[i];
+    // V in LDS: [key block][16-row group j][quad][row in group][4 keys], so that the 64
+    // lanes of an A-operand read (lane = quad*16 + row) touch 512 consecutive bytes
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
-      const int chunk = i * (kWaves * 64) + tid;
-      *reinterpret_cast<uint4*>(v_lds + chunk * 8) = vreg[i];
+      int kbi, rem;
+      if constexpr (D == 128) {
+        kbi = i;
+        rem = tid;
+      } else {
+        kbi = 2 * i + (tid >> 7);
+        rem = tid & 127;
+      }
+      const int drow = rem >> 1;
+      const int half = rem & 1;
+      bf16_t* dst = v_lds + (((kbi * NJ + (drow >> 4)) * 4 + 2 * half) * 16 + (drow & 15)) * 4;
+      *reinterpret_cast<uint2*>(dst) = make_uint2(vreg[i].x, vreg[i].y);
+      *reinterpret_cast<uint2*>(dst + 64) = make_uint2(vreg[i].z, vreg[i].w);
     }
     __syncthreads();
+    if (kb0 + kKeyBlocks < kb_end) fetch_tile(kb0 + kKeyBlocks);  // in flight while this tile is used
 
     // ---- scores of the tile for this wave's rows
     if (kb0 * 16 > wave_pos_hi) continue;  // nothing here is visible to this wave (uniform)
@@ -205,53 +274,70 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_attention_kernel(
 #pragma unroll
         for (int c = 0; c < NC; ++c)
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], qb[ct][c], acc, 0, 0, 0);
-        s[ct][kbi] = acc;
+        s[ct][kbi] = acc * scale_log2e;
       }
     }
-    // ---- softmax update per row over the 64 keys of the tile
+    // ---- softmax update per row over the 64 keys of the tile; a tile that every live row of
+    // the wave sees whole needs no masks
+    const bool whole = (kb0 + kKeyBlocks) * 16 - 1 <= wave_pos_lo && kb0 * 16 >= wave_first_hi;
+    // The reference maximum of a row only moves when the tile's maximum exceeds it by more
+    // than 2^8: probabilities then stay below 256, which bfloat16 and the float32 sums hold
+    // easily, and the running output is rescaled rarely instead of at every tile.
     s16x4_t pb[CT][kKeyBlocks];
-    float alpha[CT];
+    float mx[CT];
     bool moved = false;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
-      float mx = -INFINITY;
+      if (!whole) {
 #pragma unroll
-      for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
+        for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = (kb0 + kbi) * 16 + 4 * quad + i;
-          const bool ok = key >= my_first[ct] && key <= my_pos[ct];
-          const float v = ok ? s[ct][kbi][i] * scale_log2e : -INFINITY;
-          s[ct][kbi][i] = v;
-          mx = fmaxf(mx, v);
+          for (int i = 0; i < 4; ++i) {
+            const int key = (kb0 + kbi) * 16 + 4 * quad + i;
+            const bool ok = key >= my_first[ct] && key <= my_pos[ct];
+            s[ct][kbi][i] = ok ? s[ct][kbi][i] : -INFINITY;
+          }
         }
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[ct], mx);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      alpha[ct] = __builtin_amdgcn_exp2f(m[ct] - m_safe);
-      moved = moved || (m_new != m[ct]);
-      float ps = 0.f;
+      float v = -INFINITY;
 #pragma unroll
-      for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
+      for (int kbi = 0; kbi < kKeyBlocks; ++kbi)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float p = __builtin_amdgcn_exp2f(s[ct][kbi][i] - m_safe);
-          ps += p;
-          pb[ct][kbi][i] = static_cast<short>(f32_to_bf16_bits(p));
-        }
-      }
-      ps += __shfl_xor(ps, 16, 64);
-      ps += __shfl_xor(ps, 32, 64);
-      l[ct] = l[ct] * alpha[ct] + ps;
-      m[ct] = m_new;
+        for (int i = 0; i < 4; ++i) v = fmaxf(v, s[ct][kbi][i]);
+      v = fmaxf(v, __shfl_xor(v, 16, 64));
+      v = fmaxf(v, __shfl_xor(v, 32, 64));
+      mx[ct] = v;
+      moved = moved || (v > m[ct] + 8.f);  // also true for the first visible key (m = -inf)
     }
     if (__any(moved)) {
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
+      for (int ct = 0; ct < CT; ++ct) {
+        if (mx[ct] > m[ct] + 8.f) {
+          const float alpha = __builtin_amdgcn_exp2f(m[ct] - mx[ct]);  // 0 when m was -inf
+          m[ct] = mx[ct];
+          l[ct] *= alpha;
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) o_acc[ct][j] = o_acc[ct][j] * alpha[ct];
+          for (int j = 0; j < NJ; ++j) o_acc[ct][j] = o_acc[ct][j] * alpha;
+        }
+      }
+    }
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const float m_safe = (m[ct] == -INFINITY) ? 0.f : m[ct];
+      float ps = 0.f;
+#pragma unroll
+      for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
+        float p[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          p[i] = __builtin_amdgcn_exp2f(s[ct][kbi][i] - m_safe);
+          ps += p[i];
+        }
+        pb[ct][kbi] = pack_bf16x4(p);
+      }
+      ps += __shfl_xor(ps, 16, 64);
+      ps += __shfl_xor(ps, 32, 64);
+      l[ct] += ps;
     }
     // ---- O^T += V^T P^T
 #pragma unroll
@@ -259,7 +345,7 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_attention_kernel(
       if ((kb0 + kbi) * 16 > wave_pos_hi) break;  // uniform: later blocks weigh nothing
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const s16x4_t va = *reinterpret_cast<const s16x4_t*>(v_lds + (kbi * D + 16 * j + col) * 16 + 4 * quad);
+        const s16x4_t va = *reinterpret_cast<const s16x4_t*>(v_lds + (((kbi * NJ + j) * 4 + quad) * 16 + col) * 4);
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
           o_acc[ct][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb[ct][kbi], o_acc[ct][j], 0, 0, 0);
@@ -275,10 +361,8 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_attention_kernel(
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const f32x4_t v = o_acc[ct][j] * inv;
-      uint2 packed;
-      packed.x = f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16);
-      packed.y = f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16);
-      *reinterpret_cast<uint2*>(op + 16 * j) = packed;
+      const float vv[4] = {v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<s16x4_t*>(op + 16 * j) = pack_bf16x4(vv);
     }
   }
 }

@@ -56,7 +56,7 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v, int n_left)
   }
 }
 
-template <int RT, int NT, typename OutT>
+template <int RT, int NT, int U, typename OutT>
 __global__ void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restrict__ A,
                                    const bf16_t* __restrict__ W, const bf16_t* __restrict__ bias,
                                    int M, int N, int K, int64_t lda, int64_t ldc, int k_per_wave) {
@@ -93,7 +93,7 @@ __global__ void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restric
   // whole 32-wide steps first (no predicates, so the loads of several steps overlap), then
   // one guarded step for a tail that is a multiple of 8
   const int k_full = k_begin + ((k_end - k_begin) / 32) * 32;
-#pragma unroll 2
+#pragma unroll U
   for (int k = k_begin; k < k_full; k += 32) {
     bf16x8_t a[RT], b[NT];
 #pragma unroll
@@ -160,11 +160,11 @@ __global__ void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restric
   }
 }
 
-template <int RT, int NT, typename OutT>
+template <int RT, int NT, int U, typename OutT>
 void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
             int64_t lda, int64_t ldc, int waves, int k_per_wave, hipStream_t stream) {
   const size_t lds = static_cast<size_t>(waves - 1) * RT * NT * 64 * 4 * sizeof(float);
-  hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, OutT>), dim3((N + 16 * RT - 1) / (16 * RT)),
+  hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, U, OutT>), dim3((N + 16 * RT - 1) / (16 * RT)),
                      dim3(waves * 64), lds, stream, C, A, W, bias, M, N, K, lda, ldc, k_per_wave);
 }
 
@@ -177,6 +177,9 @@ inline void pick_shape(int N, int K, int* rt_out, int* waves_out) {
   if (N >= 16384) {
     rt = 4;
     waves = 4;
+  } else if (N > 4096) {
+    rt = 2;
+    waves = 8;
   } else {
     while (waves < 16 && K / (waves * 2) >= 128) waves *= 2;
   }
@@ -195,8 +198,17 @@ int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int 
   if ((waves - 1) * rt * nt * 1024 > 65536) return kvc_fail("kvc_gemm_skinny_bf16: launch shape needs too much LDS");
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 31) / 32 * 32;
-#define KVC_SKINNY(RT_, NT_) \
-  launch<RT_, NT_, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream)
+  int unroll = (rt == 1) ? 8 : (rt == 2 ? 4 : 2);
+  if (const char* e = getenv("KVC_SKINNY_UNROLL")) unroll = atoi(e);
+#define KVC_SKINNY(RT_, NT_)                                                                      \
+  do {                                                                                            \
+    if (unroll >= 8 && RT_ * NT_ <= 4)                                                            \
+      launch<RT_, NT_, 8, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream);     \
+    else if (unroll >= 4 && RT_ * NT_ <= 8)                                                       \
+      launch<RT_, NT_, 4, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream);     \
+    else                                                                                          \
+      launch<RT_, NT_, 2, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream);     \
+  } while (0)
   const int key = rt * 10 + nt;
   switch (key) {
     case 11: KVC_SKINNY(1, 1); break;
