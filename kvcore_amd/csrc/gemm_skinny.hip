@@ -56,8 +56,8 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v, int n_left)
   }
 }
 
-template <int RT, int NT, int U, typename OutT>
-__global__ void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restrict__ A,
+template <int RT, int NT, int U, int MAXW, typename OutT>
+__global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restrict__ A,
                                    const bf16_t* __restrict__ W, const bf16_t* __restrict__ bias,
                                    int M, int N, int K, int64_t lda, int64_t ldc, int k_per_wave) {
   extern __shared__ float red[];  // [waves - 1][RT * NT][64][4]
@@ -90,11 +90,51 @@ __global__ void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restric
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // whole 32-wide steps first (no predicates, so the loads of several steps overlap), then
-  // one guarded step for a tail that is a multiple of 8
-  const int k_full = k_begin + ((k_end - k_begin) / 32) * 32;
-#pragma unroll U
-  for (int k = k_begin; k < k_full; k += 32) {
+  // Whole steps of 64 along K first, software-pipelined: the loads of step i+1 are issued
+  // before the products of step i, so every wave always has a step's worth of 16-byte
+  // loads in flight (a lane reads 2 x 16 bytes = a row reads 128 contiguous bytes a
+  // step).  Then whole 32-wide steps, then one guarded step for a tail (a multiple of 8).
+  constexpr int STAGES = U;  // steps in flight, the one being multiplied included
+  bf16x8_t abuf[STAGES][RT][2], bbuf[STAGES][NT][2];
+  auto load_step = [&](int stage, int k) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      abuf[stage][rt][0] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k);
+      abuf[stage][rt][1] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k + 32);
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      bbuf[stage][nt][0] = *reinterpret_cast<const bf16x8_t*>(ap[nt] + k);
+      bbuf[stage][nt][1] = *reinterpret_cast<const bf16x8_t*>(ap[nt] + k + 32);
+    }
+  };
+  auto mma_step = [&](int stage) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(abuf[stage][rt][h], bbuf[stage][nt][h],
+                                                                 acc[rt][nt], 0, 0, 0);
+  };
+  const int n64 = (k_end - k_begin) / 64;
+  int k = k_begin;
+#pragma unroll
+  for (int st = 0; st < STAGES - 1; ++st)
+    if (st < n64) load_step(st, k_begin + 64 * st);
+  for (int i = 0; i < n64; i += STAGES) {
+#pragma unroll
+    for (int j = 0; j < STAGES; ++j) {
+      if (i + j < n64) {  // uniform
+        if (i + j + STAGES - 1 < n64) load_step((j + STAGES - 1) % STAGES, k_begin + 64 * (i + j + STAGES - 1));
+        mma_step(j);
+      }
+    }
+  }
+  k = k_begin + 64 * n64;
+  const int k_full = k + ((k_end - k) / 32) * 32;
+  for (; k < k_full; k += 32) {
     bf16x8_t a[RT], b[NT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) a[rt] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k);
@@ -160,31 +200,38 @@ __global__ void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restric
   }
 }
 
-template <int RT, int NT, int U, typename OutT>
+template <int RT, int NT, typename OutT>
 void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
             int64_t lda, int64_t ldc, int waves, int k_per_wave, hipStream_t stream) {
+  // steps in flight by what fits in registers beside the accumulators
+  constexpr int STAGES = (RT + NT <= 5) ? 4 : ((RT + NT <= 6) ? 3 : 2);
+  constexpr int MAXW = (RT >= 2) ? 4 : 8;
   const size_t lds = static_cast<size_t>(waves - 1) * RT * NT * 64 * 4 * sizeof(float);
-  hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, U, OutT>), dim3((N + 16 * RT - 1) / (16 * RT)),
-                     dim3(waves * 64), lds, stream, C, A, W, bias, M, N, K, lda, ldc, k_per_wave);
+  hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, STAGES, MAXW, OutT>),
+                     dim3((N + 16 * RT - 1) / (16 * RT)), dim3(waves * 64), lds, stream, C, A, W,
+                     bias, M, N, K, lda, ldc, k_per_wave);
 }
 
 // The launch shape is a function of N and K alone, so that a row's sums do not depend on
-// how many rows come with it.  KVC_SKINNY_RT / KVC_SKINNY_WAVES override it for tuning.
+// how many rows come with it.  Measured on MI355X at 1 to 16 rows: outputs wider than 4096
+// want 32 weight rows a wave and 4 waves along K, narrower ones 16 rows and 8 waves.
+// KVC_SKINNY_RT / KVC_SKINNY_WAVES override the choice for tuning.
 inline void pick_shape(int N, int K, int* rt_out, int* waves_out) {
-  // measured on MI355X at M = 1 and 8: wide outputs want 64 rows a block and 4 waves along
-  // K, narrow ones 16 rows and as many waves as K allows
-  int rt = 1, waves = 1;
-  if (N >= 16384) {
-    rt = 4;
-    waves = 4;
-  } else if (N > 4096) {
+  int rt, waves;
+  if (N > 4096) {
     rt = 2;
-    waves = 8;
+    waves = 4;
   } else {
-    while (waves < 16 && K / (waves * 2) >= 128) waves *= 2;
+    rt = 1;
+    waves = 8;
   }
+  while (waves > 1 && K / waves < 128) waves /= 2;
   if (const char* e = getenv("KVC_SKINNY_RT")) rt = atoi(e);
   if (const char* e = getenv("KVC_SKINNY_WAVES")) waves = atoi(e);
+  if (rt != 1 && rt != 2) rt = 1;
+  const int max_waves = (rt >= 2) ? 4 : 8;
+  if (waves < 1) waves = 1;
+  if (waves > max_waves) waves = max_waves;
   *rt_out = rt;
   *waves_out = waves;
 }
@@ -195,31 +242,17 @@ int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int 
   int rt, waves;
   pick_shape(N, K, &rt, &waves);
   const int nt = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
-  if ((waves - 1) * rt * nt * 1024 > 65536) return kvc_fail("kvc_gemm_skinny_bf16: launch shape needs too much LDS");
   int k_per_wave = (K + waves - 1) / waves;
-  k_per_wave = (k_per_wave + 31) / 32 * 32;
-  int unroll = (rt == 1) ? 8 : (rt == 2 ? 4 : 2);
-  if (const char* e = getenv("KVC_SKINNY_UNROLL")) unroll = atoi(e);
-#define KVC_SKINNY(RT_, NT_)                                                                      \
-  do {                                                                                            \
-    if (unroll >= 8 && RT_ * NT_ <= 4)                                                            \
-      launch<RT_, NT_, 8, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream);     \
-    else if (unroll >= 4 && RT_ * NT_ <= 8)                                                       \
-      launch<RT_, NT_, 4, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream);     \
-    else                                                                                          \
-      launch<RT_, NT_, 2, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream);     \
-  } while (0)
-  const int key = rt * 10 + nt;
-  switch (key) {
+  k_per_wave = (k_per_wave + 63) / 64 * 64;
+#define KVC_SKINNY(RT_, NT_) \
+  launch<RT_, NT_, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream)
+  switch (rt * 10 + nt) {
     case 11: KVC_SKINNY(1, 1); break;
     case 12: KVC_SKINNY(1, 2); break;
     case 14: KVC_SKINNY(1, 4); break;
     case 21: KVC_SKINNY(2, 1); break;
     case 22: KVC_SKINNY(2, 2); break;
     case 24: KVC_SKINNY(2, 4); break;
-    case 41: KVC_SKINNY(4, 1); break;
-    case 42: KVC_SKINNY(4, 2); break;
-    case 44: KVC_SKINNY(4, 4); break;
     default: return kvc_fail("kvc_gemm_skinny_bf16: unsupported launch shape");
   }
 #undef KVC_SKINNY

@@ -364,9 +364,10 @@ def linear(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tens
     N = w.shape[0]
     skinny_ok = (M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0
                  and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
-    # measured on MI355X: the weight-streaming kernel wins for up to 16 rows unless K or N
-    # is very large; it is also the only one that stores float32
-    if skinny_ok and (out.dtype == torch.float32
+    # measured on MI355X (N x K of 4096..128256 x 4096..14336): the weight-streaming kernel
+    # wins up to 8 rows everywhere and up to 16 rows unless K or N is very large; it is also
+    # the only one that stores float32
+    if skinny_ok and (out.dtype == torch.float32 or M <= 8
                       or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)):
         gemm_skinny_bf16(out, x, w, bias)
         return

@@ -45,7 +45,8 @@ class OutputHead(Part):
             ops.linear(logits, hidden_rows, w)
             return
         S = hidden_rows.shape[0]
-        if S <= ops.SKINNY_PREFERRED_ROWS and self.vocab_size < 65536 and self.hidden_size % 8 == 0:
+        if self.hidden_size % 8 == 0 and (S <= 8 or (S <= ops.SKINNY_PREFERRED_ROWS
+                                                      and self.vocab_size < 65536)):
             ops.linear(logits, hidden_rows, w)  # float32 sums are stored without rounding
             return
         low = ctx.buffers.get("head_logits_dt", S, self.vocab_size, hidden_rows.dtype)
