@@ -378,73 +378,129 @@ extern "C" int kvc_rope_table(float* cos_out, float* sin_out, const int32_t* pos
   return kvc_check_launch("kvc_rope_table");
 }
 
+// ------------------------------------------------------------------ cache slots
+// kv_slot[t] = page * page_size + position % page_size of token t in its request's block
+// table row; -1 when the table has no page there; -2 for a padding token.
+__global__ void kv_slots_kernel(int32_t* __restrict__ kv_slot, const int32_t* __restrict__ positions,
+                                const int32_t* __restrict__ token_req,
+                                const int32_t* __restrict__ slots, const int32_t* __restrict__ table,
+                                int table_stride, int T, int page_size, int num_pages) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const int req = token_req[t];
+  if (req < 0) {
+    kv_slot[t] = -2;
+    return;
+  }
+  const int pos = positions[t];
+  const int idx = pos / page_size;
+  int out = -1;
+  if (idx < table_stride) {
+    const int page = table[static_cast<int64_t>(slots[req]) * table_stride + idx];
+    if (page > 0 && page < num_pages) out = page * page_size + pos % page_size;
+  }
+  kv_slot[t] = out;
+}
+
+extern "C" int kvc_kv_slots(int32_t* kv_slot, const int32_t* positions, const int32_t* token_req,
+                            const int32_t* slots, const int32_t* table, int table_stride, int T,
+                            int page_size, int num_pages, kvc_stream stream) {
+  if (T < 0 || table_stride <= 0 || page_size <= 0 || num_pages <= 0)
+    return kvc_fail("kvc_kv_slots: bad sizes");
+  if (static_cast<int64_t>(num_pages) * page_size > 0x7fffffffLL)
+    return kvc_fail("kvc_kv_slots: cache too large for 32-bit slots");
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(kv_slots_kernel, dim3((T + 255) / 256), dim3(256), 0, S(stream), kv_slot,
+                     positions, token_req, slots, table, table_stride, T, page_size, num_pages);
+  return kvc_check_launch("kvc_kv_slots");
+}
+
 // ------------------------------------------------- rotation fused with the K/V write
 // One block per token.  Work items: (head, pair) rotations for the nh + nkv rotated
-// heads, then pass-through elements (beyond rot_dim, and all of v).
-template <typename T>
+// heads, then pass-through elements (beyond rot_dim, and all of v).  K pages are
+// [kv head, page_size, d]; V pages are [kv head, d, page_size] (keys contiguous).
+// VEC = 8 handles eight pairs per item with 16-byte accesses (half-split pairing, rot_dim
+// a multiple of 16); VEC = 1 is the general path.
+template <typename T, int VEC>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cache,
                                      T* __restrict__ v_cache, const float* __restrict__ cos_tab,
                                      const float* __restrict__ sin_tab, int rot_dim,
-                                     int interleaved, const int32_t* __restrict__ positions,
-                                     const int32_t* __restrict__ token_req,
-                                     const int32_t* __restrict__ slots,
-                                     const int32_t* __restrict__ table, int table_stride, int nh,
-                                     int nkv, int d, int page_size, int num_pages, int write_kv) {
+                                     int interleaved, const int32_t* __restrict__ kv_slot, int nh,
+                                     int nkv, int d, int page_size, int write_kv) {
   const int t = blockIdx.x;
-  const int req = token_req[t];
-  if (req < 0) return;
-  const int pos = positions[t];
+  const int slot = kv_slot[t];
+  if (slot == -2) return;  // padding token
   const int half = rot_dim / 2;
   T* row = qkv + static_cast<int64_t>(t) * (nh + 2 * nkv) * d;
 
-  // K pages are [kv head, page_size, d]; V pages are [kv head, d, page_size] (keys contiguous)
-  int64_t cache_base = -1;  // element offset of K[page, kv head 0, pos % page_size, 0]
-  int64_t v_base = -1;      // element offset of V[page, kv head 0, 0, pos % page_size]
-  if (write_kv) {
-    const int slot = slots[req];
-    const int page = table[static_cast<int64_t>(slot) * table_stride + pos / page_size];
-    if (page > 0 && page < num_pages) {
-      cache_base = (static_cast<int64_t>(page) * nkv * page_size + pos % page_size) * d;
-      v_base = static_cast<int64_t>(page) * nkv * page_size * d + pos % page_size;
-    }
+  int64_t k_base = -1, v_base = -1;
+  if (write_kv && slot >= 0) {
+    const int page = slot / page_size, off = slot - page * page_size;
+    k_base = (static_cast<int64_t>(page) * nkv * page_size + off) * d;       // K[page, 0, off, 0]
+    v_base = static_cast<int64_t>(page) * nkv * page_size * d + off;         // V[page, 0, 0, off]
   }
   const int64_t head_step = static_cast<int64_t>(page_size) * d;  // between kv heads in a page
-
   const float* cs = cos_tab + static_cast<int64_t>(t) * half;
   const float* sn = sin_tab + static_cast<int64_t>(t) * half;
 
-  // rotations: heads 0..nh-1 are q, nh..nh+nkv-1 are k
-  const int n_rot = (nh + nkv) * half;
-  for (int w = threadIdx.x; w < n_rot; w += blockDim.x) {
-    const int head = w / half;
-    const int j = w - head * half;
-    const int i0 = interleaved ? 2 * j : j;
-    const int i1 = interleaved ? 2 * j + 1 : j + half;
-    T* hp = row + static_cast<int64_t>(head) * d;
-    const float x0 = to_float(hp[i0]);
-    const float x1 = to_float(hp[i1]);
-    const float c = cs[j], s = sn[j];
-    const T y0 = from_float<T>(x0 * c - x1 * s);
-    const T y1 = from_float<T>(x1 * c + x0 * s);
-    hp[i0] = y0;
-    hp[i1] = y1;
-    if (head >= nh && cache_base >= 0) {
-      T* kc = k_cache + cache_base + (head - nh) * head_step;
-      kc[i0] = y0;
-      kc[i1] = y1;
+  if constexpr (VEC == 8) {
+    const int chunks = half / 8;
+    const int n_items = (nh + nkv) * chunks;
+    for (int w = threadIdx.x; w < n_items; w += blockDim.x) {
+      const int head = w / chunks;
+      const int j = (w - head * chunks) * 8;
+      T* hp = row + static_cast<int64_t>(head) * d;
+      float x0[8], x1[8], c[8], s_[8], y0[8], y1[8];
+      load8(hp + j, x0);
+      load8(hp + j + half, x1);
+      load8(cs + j, c);
+      load8(sn + j, s_);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        y0[e] = x0[e] * c[e] - x1[e] * s_[e];
+        y1[e] = x1[e] * c[e] + x0[e] * s_[e];
+      }
+      store8(hp + j, y0);
+      store8(hp + j + half, y1);
+      if (head >= nh && k_base >= 0) {
+        T* kc = k_cache + k_base + (head - nh) * head_step;
+        store8(kc + j, y0);
+        store8(kc + j + half, y1);
+      }
+    }
+  } else {
+    const int n_rot = (nh + nkv) * half;
+    for (int w = threadIdx.x; w < n_rot; w += blockDim.x) {
+      const int head = w / half;
+      const int j = w - head * half;
+      const int i0 = interleaved ? 2 * j : j;
+      const int i1 = interleaved ? 2 * j + 1 : j + half;
+      T* hp = row + static_cast<int64_t>(head) * d;
+      const float x0 = to_float(hp[i0]);
+      const float x1 = to_float(hp[i1]);
+      const float c = cs[j], s_ = sn[j];
+      const T y0 = from_float<T>(x0 * c - x1 * s_);
+      const T y1 = from_float<T>(x1 * c + x0 * s_);
+      hp[i0] = y0;
+      hp[i1] = y1;
+      if (head >= nh && k_base >= 0) {
+        T* kc = k_cache + k_base + (head - nh) * head_step;
+        kc[i0] = y0;
+        kc[i1] = y1;
+      }
     }
   }
-  if (cache_base < 0) return;
+  if (k_base < 0) return;
   // k elements beyond the rotated part
   const int tail = d - rot_dim;
   if (tail > 0) {
     for (int w = threadIdx.x; w < nkv * tail; w += blockDim.x) {
       const int head = w / tail;
       const int i = rot_dim + (w - head * tail);
-      k_cache[cache_base + head * head_step + i] = row[static_cast<int64_t>(nh + head) * d + i];
+      k_cache[k_base + head * head_step + i] = row[static_cast<int64_t>(nh + head) * d + i];
     }
   }
-  // v
+  // v, element i of a head goes to V[page, head, i, off]
   for (int w = threadIdx.x; w < nkv * d; w += blockDim.x) {
     const int head = w / d;
     const int i = w - head * d;
@@ -455,22 +511,31 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
 
 extern "C" int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_tab,
                                  const float* sin_tab, int rot_dim, int interleaved,
-                                 const int32_t* positions, const int32_t* token_req,
-                                 const int32_t* slots, const int32_t* table, int table_stride,
-                                 int T, int nh, int nkv, int d, int page_size, int num_pages,
-                                 int write_kv, int dtype, kvc_stream stream) {
-  if (T < 0 || nh <= 0 || nkv <= 0 || d <= 0 || page_size <= 0 || num_pages <= 0)
+                                 const int32_t* kv_slot, int T, int nh, int nkv, int d,
+                                 int page_size, int write_kv, int dtype, kvc_stream stream) {
+  if (T < 0 || nh <= 0 || nkv <= 0 || d <= 0 || page_size <= 0)
     return kvc_fail("kvc_rope_kv_write: bad sizes");
   if (rot_dim < 0 || rot_dim > d || (rot_dim & 1))
     return kvc_fail("kvc_rope_kv_write: rot_dim must be even and at most the head size");
   if (T == 0) return 0;
-  KVC_DISPATCH_DTYPE(
-      dtype, Tp,
-      hipLaunchKernelGGL(rope_kv_write_kernel<Tp>, dim3(T), dim3(256), 0, S(stream),
-                         static_cast<Tp*>(qkv), static_cast<Tp*>(k_cache),
-                         static_cast<Tp*>(v_cache), cos_tab, sin_tab, rot_dim, interleaved,
-                         positions, token_req, slots, table, table_stride, nh, nkv, d, page_size,
-                         num_pages, write_kv));
+  const auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const bool vec = !interleaved && rot_dim > 0 && rot_dim % 16 == 0 && d % 8 == 0 &&
+                   aligned16(qkv) && aligned16(k_cache) && aligned16(cos_tab) && aligned16(sin_tab);
+  if (vec) {
+    KVC_DISPATCH_DTYPE(
+        dtype, Tp,
+        hipLaunchKernelGGL((rope_kv_write_kernel<Tp, 8>), dim3(T), dim3(256), 0, S(stream),
+                           static_cast<Tp*>(qkv), static_cast<Tp*>(k_cache),
+                           static_cast<Tp*>(v_cache), cos_tab, sin_tab, rot_dim, interleaved,
+                           kv_slot, nh, nkv, d, page_size, write_kv));
+  } else {
+    KVC_DISPATCH_DTYPE(
+        dtype, Tp,
+        hipLaunchKernelGGL((rope_kv_write_kernel<Tp, 1>), dim3(T), dim3(256), 0, S(stream),
+                           static_cast<Tp*>(qkv), static_cast<Tp*>(k_cache),
+                           static_cast<Tp*>(v_cache), cos_tab, sin_tab, rot_dim, interleaved,
+                           kv_slot, nh, nkv, d, page_size, write_kv));
+  }
   return kvc_check_launch("kvc_rope_kv_write");
 }
 

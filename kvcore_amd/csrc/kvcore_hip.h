@@ -48,18 +48,23 @@ int kvc_to_float(float* out, const void* in, int64_t n, int dtype, kvc_stream st
 int kvc_rope_table(float* cos_out, float* sin_out, const int32_t* positions,
                    const float* inv_freq, int T, int half, kvc_stream stream);
 
+// kv_slot[t] = page * page_size + position % page_size, where page = table[slots[
+// token_req[t]], position / page_size]; -1 when the table holds no page there, -2 for a
+// padding token (token_req < 0).
+int kvc_kv_slots(int32_t* kv_slot, const int32_t* positions, const int32_t* token_req,
+                 const int32_t* slots, const int32_t* table, int table_stride, int T,
+                 int page_size, int num_pages, kvc_stream stream);
+
 // Rotates the first rot_dim elements of every q and k head of qkv [T, (nh+2nkv)*d] in
 // place (pairs (j, j+rot_dim/2), or (2j, 2j+1) when interleaved), then, when write_kv is
-// set, stores the rotated k and the v of token t at its page slot:
-//   slot row  = slots[token_req[t]], page = table[row, pos / page_size],
-//   k_cache[page, kv_head, pos % page_size, :] and v_cache[page, kv_head, :, pos % page_size]
+// set and kv_slot[t] >= 0, stores the rotated k and the v of token t at that slot:
+//   k_cache[page, kv_head, offset, :] and v_cache[page, kv_head, :, offset]
 //   (V pages keep the keys contiguous: the layout the matrix cores read).
-// Tokens with token_req < 0 are left alone.
+// Tokens with kv_slot == -2 are left alone.
 int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_tab,
-                      const float* sin_tab, int rot_dim, int interleaved,
-                      const int32_t* positions, const int32_t* token_req, const int32_t* slots,
-                      const int32_t* table, int table_stride, int T, int nh, int nkv, int d,
-                      int page_size, int num_pages, int write_kv, int dtype, kvc_stream stream);
+                      const float* sin_tab, int rot_dim, int interleaved, const int32_t* kv_slot,
+                      int T, int nh, int nkv, int d, int page_size, int write_kv, int dtype,
+                      kvc_stream stream);
 
 // Attention of every token over its request's cache: token t at position p sees keys
 // max(0, p - window + 1) .. p (window <= 0: all), read through the block table.
@@ -72,8 +77,11 @@ int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* 
 
 // The same attention for bfloat16 on the matrix cores, one wave per (token, kv head,
 // split): meant for steps of single tokens.  nsplit > 1 needs part_o [T, nh, nsplit, d]
-// and part_ml [T, nh, nsplit, 2] float32.  kvc_decode_attention_supported tells whether
-// a shape is served (else use kvc_paged_attention).
+// and part_ml [T, nh, nsplit, 2] float32; a second kernel combines the splits (a "last
+// wave combines" scheme needs device-scope fences, which on this chip write back and
+// invalidate a whole L2 slice per wave and cost more than the launch they save).
+// kvc_decode_attention_supported tells whether a shape is served (else use
+// kvc_paged_attention).
 int kvc_decode_attention_supported(int nh, int nkv, int d, int page_size, int dtype);
 int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* q, int64_t q_stride,
                          const void* k_cache, const void* v_cache, const int32_t* table,
@@ -107,9 +115,11 @@ int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias
 int kvc_table_update(int32_t* table, int table_stride, int table_rows, const int32_t* triples,
                      int n, kvc_stream stream);
 
-// out[s] = index of the largest logit of row s (the lowest index among equals).
+// out[s] = index of the largest logit of row s (the lowest index among equals).  With a
+// workspace (part_val, part_idx: part_capacity >= S * ceil(V / 8192) entries each) long rows
+// are searched by several blocks; the pointers may be null.
 int kvc_argmax(int32_t* out, const float* logits, int S, int V, int64_t row_stride,
-               kvc_stream stream);
+               float* part_val, int32_t* part_idx, int part_capacity, kvc_stream stream);
 
 // Per row s: temperature[s] < 1e-5 gives the argmax; otherwise
 // argmax_v(logits[v] / temperature - log(e_v)), e_v exponential noise keyed by

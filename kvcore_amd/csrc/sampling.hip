@@ -96,6 +96,43 @@ __global__ __launch_bounds__(kThreads) void argmax_kernel(int32_t* __restrict__ 
   if (threadIdx.x == 0) out[blockIdx.x] = total.idx < 0 ? 0 : total.idx;
 }
 
+// Two-stage argmax for long rows: stage one takes the best of a chunk of the row per
+// block, stage two the best of the chunk results (same order of preference: larger value,
+// then lower index).
+__global__ __launch_bounds__(kThreads) void argmax_chunk_kernel(float* __restrict__ part_val,
+                                                                int32_t* __restrict__ part_idx,
+                                                                const float* __restrict__ logits,
+                                                                int V, int64_t row_stride,
+                                                                int chunk) {
+  __shared__ Best scratch[kThreads / kWave];
+  const float* row = logits + static_cast<int64_t>(blockIdx.x) * row_stride;
+  const int begin = blockIdx.y * chunk;
+  const int end = (begin + chunk < V) ? begin + chunk : V;
+  Best mine{-INFINITY, -1};
+  for (int v = begin + threadIdx.x; v < end; v += kThreads) mine = better(mine, Best{row[v], v});
+  const Best total = block_best(mine, scratch);
+  if (threadIdx.x == 0) {
+    part_val[blockIdx.x * gridDim.y + blockIdx.y] = total.val;
+    part_idx[blockIdx.x * gridDim.y + blockIdx.y] = total.idx;
+  }
+}
+
+__global__ void argmax_final_kernel(int32_t* __restrict__ out, const float* __restrict__ part_val,
+                                    const int32_t* __restrict__ part_idx, int chunks) {
+  const int s = blockIdx.x;
+  Best mine{-INFINITY, -1};
+  for (int c = threadIdx.x; c < chunks; c += kWave)
+    mine = better(mine, Best{part_val[s * chunks + c], part_idx[s * chunks + c]});
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    Best other;
+    other.val = __shfl_xor(mine.val, o, kWave);
+    other.idx = __shfl_xor(mine.idx, o, kWave);
+    mine = better(mine, other);
+  }
+  if (threadIdx.x == 0) out[s] = mine.idx < 0 ? 0 : mine.idx;
+}
+
 __global__ __launch_bounds__(kThreads) void sample_kernel(
     int32_t* __restrict__ out, const float* __restrict__ logits, int V, int64_t row_stride,
     const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
@@ -178,9 +215,21 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(
 }  // namespace
 
 extern "C" int kvc_argmax(int32_t* out, const float* logits, int S_, int V, int64_t row_stride,
+                          float* part_val, int32_t* part_idx, int part_capacity,
                           kvc_stream stream) {
   if (S_ < 0 || V <= 0 || row_stride < V) return kvc_fail("kvc_argmax: bad sizes");
   if (S_ == 0) return 0;
+  constexpr int kChunk = 8192;
+  const int chunks = (V + kChunk - 1) / kChunk;
+  if (chunks > 1 && part_val != nullptr && part_idx != nullptr && part_capacity >= S_ * chunks &&
+      chunks <= 65535) {
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(argmax_chunk_kernel, dim3(S_, chunks), dim3(kThreads), 0, st, part_val,
+                       part_idx, logits, V, row_stride, kChunk);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(S_), dim3(kWave), 0, st, out, part_val, part_idx,
+                       chunks);
+    return kvc_check_launch("kvc_argmax");
+  }
   hipLaunchKernelGGL(argmax_kernel, dim3(S_), dim3(kThreads), 0,
                      reinterpret_cast<hipStream_t>(stream), out, logits, V, row_stride);
   return kvc_check_launch("kvc_argmax");

@@ -18,7 +18,9 @@ input_batch.py and kvcore/kv/block_table.py.  Differences that matter:
 
 from __future__ import annotations
 
+import gc
 import json
+import weakref
 from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Sequence
@@ -115,8 +117,17 @@ class ModelRunner:
             torch.zeros((max_num_seqs, *sa.need.shape), dtype=sa.need.dtype, device=self.device)
             for sa in model.state_arrays
         ]
-        self.buffers = StepBuffers(self.device, token_capacity=max_num_tokens,
-                                   on_grow=self._drop_graphs)
+        # a weak reference: the buffers must not keep the runner (its graphs and pinned
+        # memory) alive in a cycle that only the garbage collector would free, at a time
+        # of its choosing
+        self_ref = weakref.ref(self)
+
+        def drop_graphs() -> None:
+            runner = self_ref()
+            if runner is not None:
+                runner._drop_graphs()
+
+        self.buffers = StepBuffers(self.device, token_capacity=max_num_tokens, on_grow=drop_graphs)
 
         # host mirror of what each slot's table rows hold: (request id, entries synced,
         # leading entries nulled) per group
@@ -340,10 +351,18 @@ class ModelRunner:
             return run()[:num_live]
         graph = torch.cuda.CUDAGraph()
         self.buffers.frozen = True
+        # No garbage collection while the stream is capturing: a collection may free device
+        # or pinned memory or another graph that some dead object still holds, and the HIP
+        # runtime aborts the process when memory is freed during a capture.
+        gc.collect()
+        gc_was_enabled = gc.isenabled()
+        gc.disable()
         try:
             with torch.cuda.graph(graph):
                 logits = run()
         finally:
+            if gc_was_enabled:
+                gc.enable()
             self.buffers.frozen = False
         self._graphs[bucket] = (graph, logits)
         graph.replay()

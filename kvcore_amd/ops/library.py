@@ -37,7 +37,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_gather_rows": [P, P, P, I, I, I, I, P],
         "kvc_to_float": [P, P, L, I, P],
         "kvc_rope_table": [P, P, P, P, I, I, P],
-        "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
+        "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
+        "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, P],
         "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "kvc_decode_attention_supported": [I, I, I, I, I],
@@ -46,7 +47,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
         "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, P],
         "kvc_table_update": [P, I, I, P, I, P],
-        "kvc_argmax": [P, P, I, I, L, P],
+        "kvc_argmax": [P, P, I, I, L, P, P, I, P],
         "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P],
     }
     for name, argtypes in sigs.items():
@@ -189,12 +190,25 @@ def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
            "kvc_rope_table")
 
 
+def kv_slots(out: torch.Tensor, *, positions: torch.Tensor, token_req: torch.Tensor,
+             slots: torch.Tensor, table: torch.Tensor, page_size: int, num_pages: int) -> None:
+    """``out[t]`` = cache slot of token ``t`` (page * page_size + offset), -1 without a page,
+    -2 for a padding token.  Reference: kvcore/kv/block_table.py:215-227 computes the same
+    mapping per layer in Python."""
+    T = out.numel()
+    if positions.numel() < T or token_req.numel() < T:
+        raise KernelError("kv_slots: per-token arrays too short")
+    _check(load().kvc_kv_slots(_dev(out, "out", torch.int32), _dev(positions, "positions", torch.int32),
+                               _dev(token_req, "token_req", torch.int32),
+                               _dev(slots, "slots", torch.int32), _dev(table, "table", torch.int32),
+                               table.shape[1], T, page_size, num_pages, _stream()), "kvc_kv_slots")
+
+
 def rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                   cos: torch.Tensor, sin: torch.Tensor, *, rot_dim: int, interleaved: bool,
-                  positions: torch.Tensor, token_req: torch.Tensor, slots: torch.Tensor,
-                  table: torch.Tensor, nh: int, nkv: int, d: int, write_kv: bool = True) -> None:
+                  kv_slot: torch.Tensor, nh: int, nkv: int, d: int, write_kv: bool = True) -> None:
     """``k_cache`` is ``[pages, nkv, page_size, d]``, ``v_cache`` ``[pages, nkv, d, page_size]``,
-    both of the dtype of ``qkv``."""
+    both of the dtype of ``qkv``; ``kv_slot`` comes from ``kv_slots``."""
     T = qkv.shape[0]
     if qkv.shape != (T, (nh + 2 * nkv) * d):
         raise KernelError(f"rope_kv_write: qkv shape {tuple(qkv.shape)} does not fit heads")
@@ -203,15 +217,13 @@ def rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         raise KernelError("rope_kv_write: cache dtype differs from qkv")
     if cos.shape[0] < T or cos.shape[1] != rot_dim // 2 or sin.shape != cos.shape:
         raise KernelError("rope_kv_write: rotary tables do not fit")
-    if positions.numel() < T or token_req.numel() < T:
-        raise KernelError("rope_kv_write: per-token arrays too short")
+    if kv_slot.numel() < T:
+        raise KernelError("rope_kv_write: kv_slot too short")
     _check(load().kvc_rope_kv_write(
         _dev(qkv, "qkv"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), rot_dim, int(interleaved),
-        _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
-        _dev(slots, "slots", torch.int32), _dev(table, "table", torch.int32), table.shape[1],
-        T, nh, nkv, d, page_size, num_pages, int(write_kv), _code(qkv, "qkv"), _stream()),
-        "kvc_rope_kv_write")
+        _dev(kv_slot, "kv_slot", torch.int32), T, nh, nkv, d, page_size, int(write_kv),
+        _code(qkv, "qkv"), _stream()), "kvc_rope_kv_write")
 
 
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -388,12 +400,20 @@ def table_update(table: torch.Tensor, triples: torch.Tensor, n: int) -> None:
            "kvc_table_update")
 
 
-def argmax(out: torch.Tensor, logits: torch.Tensor) -> None:
+def argmax(out: torch.Tensor, logits: torch.Tensor, part_val: torch.Tensor | None = None,
+           part_idx: torch.Tensor | None = None) -> None:
+    """``part_val`` (float32) and ``part_idx`` (int32) of equal length are an optional
+    workspace that lets several blocks search one long row."""
     S, V = logits.shape
     if out.numel() < S or logits.stride(1) != 1 or logits.dtype != torch.float32 or not logits.is_cuda:
         raise KernelError("argmax: expects float32 GPU logits [S, V] and S outputs")
+    pv = pi = None
+    cap = 0
+    if part_val is not None and part_idx is not None:
+        pv, pi = _dev(part_val, "part_val", torch.float32), _dev(part_idx, "part_idx", torch.int32)
+        cap = min(part_val.numel(), part_idx.numel())
     _check(load().kvc_argmax(_dev(out, "out", torch.int32), logits.data_ptr(), S, V,
-                             logits.stride(0), _stream()), "kvc_argmax")
+                             logits.stride(0), pv, pi, cap, _stream()), "kvc_argmax")
 
 
 def sample(out: torch.Tensor, logits: torch.Tensor, *, temperature: torch.Tensor,

@@ -15,7 +15,7 @@ from kvcore_amd.ops import library as ops
 from .base import CacheNeed, Mixer, ParamSource, ParamSpec, PositionEncoding, register_mixer
 
 
-DECODE_TARGET_WAVES = 2048  # enough single-wave blocks to keep 256 compute units fed
+DECODE_TARGET_WAVES = 1024  # enough single-wave blocks to keep 256 compute units fed
 DECODE_MAX_SPLITS = 32
 
 
@@ -84,9 +84,16 @@ class PagedAttention(Mixer):
             rot_dim, interleaved = 0, False
         else:
             cos, sin, rot_dim, interleaved = rot.cos, rot.sin, rot.rot_dim, rot.interleaved
+        # where each token's key and value go: once per step and cache group
+        slot_key = ("kv_slot", call.group_index)
+        kv_slot = ctx.scratch.get(slot_key)
+        if kv_slot is None:
+            kv_slot = ctx.buf(f"kv_slot_{call.group_index}", 1, torch.int32).view(-1)
+            ops.kv_slots(kv_slot, positions=ctx.positions, token_req=ctx.token_req, slots=ctx.slots,
+                         table=group.table, page_size=group.page_size, num_pages=k_cache.shape[0])
+            ctx.scratch[slot_key] = kv_slot
         ops.rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim, interleaved=interleaved,
-                          positions=ctx.positions, token_req=ctx.token_req, slots=ctx.slots,
-                          table=group.table, nh=self.num_heads, nkv=self.num_kv_heads,
+                          kv_slot=kv_slot, nh=self.num_heads, nkv=self.num_kv_heads,
                           d=self.head_dim, write_kv=call.write_cache)
 
         attn = ctx.buf("attn_out", self.q_size)

@@ -47,6 +47,8 @@ class Sampler:
         self._dev = torch.empty(6 * n, dtype=torch.int32, device=self.device)
         self._out_dev = torch.empty(n, dtype=torch.int32, device=self.device)
         self._out_host = torch.empty(n, dtype=torch.int32, pin_memory=True)
+        self._part_val: torch.Tensor | None = None  # workspace of the two-stage argmax
+        self._part_idx: torch.Tensor | None = None
 
     def resolve_seed(self, params: SamplingParams) -> int:
         """The request's own seed, or one derived from the engine's seed and the order of
@@ -68,7 +70,11 @@ class Sampler:
             raise ValueError(f"{S} rows exceed the sampler's capacity {self.max_rows}")
         out = self._out_dev[:S]
         if all(r.params.temperature < GREEDY_EPS for r in rows):
-            ops.argmax(out, logits)
+            need = S * (-(-logits.shape[1] // 8192))
+            if self._part_val is None or self._part_val.numel() < need:
+                self._part_val = torch.empty(max(need, self.max_rows), dtype=torch.float32, device=self.device)
+                self._part_idx = torch.empty(max(need, self.max_rows), dtype=torch.int32, device=self.device)
+            ops.argmax(out, logits, self._part_val, self._part_idx)
         else:
             n = self.max_rows
             buf = self._host_np

@@ -189,7 +189,7 @@ def make_cache(pages, nkv, page_size, d, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("interleaved,rot_dim", [(False, 32), (True, 32), (False, 16), (False, 0)])
+@pytest.mark.parametrize("interleaved,rot_dim", [(False, 32), (True, 32), (False, 16), (False, 8), (False, 0)])
 def test_rope_kv_write(ops, dtype, interleaved, rot_dim):
     nh, nkv, d, page = 3, 1, 32, 4
     T = 6
@@ -208,9 +208,12 @@ def test_rope_kv_write(ops, dtype, interleaved, rot_dim):
     if rot_dim:
         ops.rope_table(cos, sin, positions, inv)
     qkv = qkv0.clone()
+    kv_slot = torch.empty(T, dtype=torch.int32, device=DEV)
+    ops.kv_slots(kv_slot, positions=positions, token_req=token_req, slots=slots, table=table,
+                 page_size=page, num_pages=7)
+    assert kv_slot.cpu().tolist() == [3 * 4 + 1, 3 * 4 + 2, 3 * 4 + 3, 1 * 4 + 0, 1 * 4 + 1, -2]
     ops.rope_kv_write(qkv, kc, vc, cos, sin, rot_dim=rot_dim, interleaved=interleaved,
-                      positions=positions, token_req=token_req, slots=slots, table=table,
-                      nh=nh, nkv=nkv, d=d)
+                      kv_slot=kv_slot, nh=nh, nkv=nkv, d=d)
 
     def rotate(x):  # x [T, heads, d] float64
         if not rot_dim:
@@ -245,10 +248,24 @@ def test_rope_kv_write(ops, dtype, interleaved, rot_dim):
     kc2, vc2 = make_cache(7, nkv, page, d, dtype)
     qkv = qkv0.clone()
     ops.rope_kv_write(qkv, kc2, vc2, cos, sin, rot_dim=rot_dim, interleaved=interleaved,
-                      positions=positions, token_req=token_req, slots=slots, table=table,
-                      nh=nh, nkv=nkv, d=d, write_kv=False)
+                      kv_slot=kv_slot, nh=nh, nkv=nkv, d=d, write_kv=False)
     assert torch.isnan(kc2).all() and torch.isnan(vc2).all()
     assert torch.allclose(qkv.double().cpu().view(T, -1, d)[live, :nh], want_q[live], **tol(dtype))
+
+
+def test_kv_slots_vector_of_the_reference(ops):
+    """tests/test_block_table.py:65-85: rows [3,4] and [5], page size 2, positions
+    [0,1,2,3,0,1] -> slots [6,7,8,9,10,11]; beyond the row's pages there is no slot."""
+    table = torch.zeros(2, 3, dtype=torch.int32, device=DEV)
+    table[0, :2] = torch.tensor([3, 4], dtype=torch.int32)
+    table[1, :1] = torch.tensor([5], dtype=torch.int32)
+    positions = torch.tensor([0, 1, 2, 3, 0, 1, 2, 0], dtype=torch.int32, device=DEV)
+    token_req = torch.tensor([0, 0, 0, 0, 1, 1, 1, -1], dtype=torch.int32, device=DEV)
+    out = torch.empty(8, dtype=torch.int32, device=DEV)
+    ops.kv_slots(out, positions=positions, token_req=token_req,
+                 slots=torch.tensor([0, 1], dtype=torch.int32, device=DEV), table=table,
+                 page_size=2, num_pages=8)
+    assert out.cpu().tolist() == [6, 7, 8, 9, 10, 11, -1, -2]
 
 
 def paged_setup(seq_lens, nkv, d, page, dtype, seed=0, shuffle=True):
@@ -572,6 +589,21 @@ def test_argmax_takes_the_lowest_index_among_equals(ops):
     wide[:, :1000] = logits
     ops.argmax(out, wide[:, :1000])
     assert out.cpu().tolist() == want
+    # long rows searched by several blocks: ties across chunk borders still go to the lowest index
+    V = 3 * 8192 + 77
+    long = rnd(5, V, seed=10)
+    long[0, 8191] = long[0, 8192] = 70.0
+    long[1, V - 1] = 70.0
+    long[2, 0] = long[2, 20000] = 70.0
+    part_val = torch.empty(5 * 4, device=DEV)
+    part_idx = torch.empty(5 * 4, dtype=torch.int32, device=DEV)
+    out5 = torch.empty(5, dtype=torch.int32, device=DEV)
+    ops.argmax(out5, long, part_val, part_idx)
+    want5 = long.cpu().argmax(-1).tolist()
+    want5[0], want5[1], want5[2] = 8191, V - 1, 0
+    assert out5.cpu().tolist() == want5
+    ops.argmax(out5, long)
+    assert out5.cpu().tolist() == want5
 
 
 @pytest.mark.parametrize("V", [331, 5000])
