@@ -170,7 +170,7 @@ def main() -> int:
     bytes_step = weight_bytes_per_step(cfg, esize) + kv_bytes(cfg, args.batch, mean_ctx, esize)
     achieved = bytes_step / sec_per_step
     result = {
-        "metric": "decode tok/s (Llama-3-8B shape, batch 8, 512-token prompts)",
+        "metric": f"decode tok/s (Llama-3-8B shape, batch {args.batch}, 512-token prompts)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

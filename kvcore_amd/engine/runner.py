@@ -154,6 +154,7 @@ class ModelRunner:
         self._np = {name: self._meta_np[o:o + n] for name, (o, n) in self._off.items()}
         self._copy_done = torch.cuda.Event()
         self._copy_pending = False
+        self._arange = np.arange(max(T, R) + 1, dtype=np.int32)
 
         # steps of single tokens are captured once per batch-size bucket and replayed
         self.use_hip_graphs = use_hip_graphs and model.graph_safe()
@@ -235,7 +236,45 @@ class ModelRunner:
         if self._copy_pending:
             self._copy_done.synchronize()
             self._copy_pending = False
-        for r, e in enumerate(entries):
+        decode_only = all(len(e.tokens) == 1 for e in entries)
+        if decode_only:
+            # single tokens only: the same checks and arrays as below, without a loop of
+            # array operations per request
+            toks = [e.tokens[0] for e in entries]
+            starts = [e.start for e in entries]
+            slot_list = [e.slot for e in entries]
+            if min(toks) < 0 or max(toks) >= vocab:
+                raise ValueError(f"a token id is outside [0, {vocab})")
+            if min(starts) < 0 or max(starts) >= self.max_model_len:
+                raise ValueError(f"a position exceeds max_model_len={self.max_model_len}")
+            if R > self.max_num_tokens:
+                raise ValueError(f"step exceeds max_num_tokens={self.max_num_tokens}")
+            if min(slot_list) < 0 or max(slot_list) >= self.max_num_seqs or len(set(slot_list)) != R:
+                raise ValueError("a slot is invalid or used twice")
+            page = self.page_size
+            for e in entries:
+                for g_pages in e.pages:
+                    if len(g_pages) * page <= e.start:
+                        raise ValueError(f"request {e.request_id!r}: {len(g_pages)} pages do not hold "
+                                         f"{e.start + 1} tokens")
+            npv["token_ids"][:R] = toks
+            npv["positions"][:R] = starts
+            npv["token_req"][:R] = self._arange[:R]
+            npv["q_start"][:R + 1] = self._arange[:R + 1]
+            npv["seq_lens"][:R] = starts
+            npv["seq_lens"][:R] += 1
+            npv["slots"][:R] = slot_list
+            for r, e in enumerate(entries):
+                for w in e.want:
+                    if w != 0:
+                        raise ValueError(f"request {e.request_id!r}: wanted index {w} outside its 1 token")
+                    npv["logit_rows"][n_rows] = r
+                    owners.append((r, e.start))
+                    n_rows += 1
+            q_lens = [1] * R
+            seq_lens = [s_ + 1 for s_ in starts]
+            t = R
+        for r, e in enumerate(entries if not decode_only else ()):
             n = len(e.tokens)
             if n == 0:
                 raise ValueError(f"request {e.request_id!r}: a step entry needs at least one token")
