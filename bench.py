@@ -30,6 +30,13 @@ LLAMA3_8B = {
     "tie_word_embeddings": False, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192,
     "hidden_act": "silu",
 }
+LLAMA32_1B = dict(LLAMA3_8B, num_hidden_layers=16, hidden_size=2048, num_attention_heads=32,
+                  num_key_value_heads=8, head_dim=64, intermediate_size=8192,
+                  rope_scaling=dict(LLAMA3_8B["rope_scaling"], factor=32.0), tie_word_embeddings=True)
+LLAMA31_70B = dict(LLAMA3_8B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+                   num_key_value_heads=8, head_dim=128, intermediate_size=28672)
+MODELS = {"8b": ("llama-3-8b-shape-random", LLAMA3_8B), "1b": ("llama-3.2-1b-shape-random", LLAMA32_1B),
+          "70b": ("llama-3.1-70b-shape-random", LLAMA31_70B)}
 CONTEXT_LEN = 8192
 PROMPT_LEN = 512
 NEW_TOKENS = 256
@@ -47,6 +54,13 @@ def parse_args():
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
     p.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    p.add_argument("--model", default="8b", choices=sorted(MODELS),
+                   help="layer sizes: 8b is the headline configuration; 1b and 70b are the other "
+                        "shapes of the baseline")
+    p.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="prompt length of the decode runs")
+    p.add_argument("--mixed", action="store_true",
+                   help="instead of the decode runs: 64 requests with prompts of 16..2048 tokens, "
+                        "portions of 512, 128 new tokens each, timed as a whole")
     p.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     p.add_argument("--only-prefill", action="store_true",
                    help="run only the 2,048-token prefill (for profiling); prints its own line")
@@ -85,7 +99,9 @@ def main() -> int:
     from kvcore_amd.engine.engine_core import EngineCore
     from kvcore_amd.engine.runner import build_model
 
-    cfg = dict(LLAMA3_8B)
+    model_name, base_cfg = MODELS[args.model]
+    cfg = dict(base_cfg)
+    prompt_len = args.prompt_len
     full_layers = cfg["num_hidden_layers"]
     if args.layers is not None:
         cfg["num_hidden_layers"] = args.layers
@@ -100,7 +116,7 @@ def main() -> int:
           f"{model.num_param_bytes() / 2**30:.2f} GiB", file=sys.stderr, flush=True)
 
     max_seqs = 64
-    pages_per_seq = -(-(PREFILL_TOKENS + NEW_TOKENS + PROMPT_LEN) // PAGE_SIZE)
+    pages_per_seq = -(-(PREFILL_TOKENS + NEW_TOKENS + prompt_len) // PAGE_SIZE)
     engine = EngineCore(KVCoreConfig(
         model_config=ModelConfig(model=".", dtype=args.dtype, max_model_len=CONTEXT_LEN),
         load_config=LoadConfig(load_format="random", seed=0),
@@ -128,16 +144,16 @@ def main() -> int:
 
     def decode_run(batch, steps, warmup):
         """tokens/s over exactly `steps` decode steps at `batch`, after `warmup` of them."""
-        slack = -(-batch * PROMPT_LEN // PREFILL_TOKENS) + 2  # steps others decode while prompts run
+        slack = -(-batch * prompt_len // PREFILL_TOKENS) + 2  # steps others decode while prompts run
         for _ in range(batch):
-            new_request(PROMPT_LEN, warmup + steps + 1 + slack)
+            new_request(prompt_len, warmup + steps + 1 + slack)
         # prompts first; a request samples its first token when its prompt ends
         while any(r.num_computed_tokens < r.num_prompt_tokens
                   for r in engine.scheduler.requests.values()):
             engine.step()
         for _ in range(warmup):
             engine.step()
-        ctx_start = PROMPT_LEN + 1 + warmup
+        ctx_start = prompt_len + 1 + warmup
         torch.cuda.synchronize()
         t_start = time.perf_counter()
         for _ in range(steps):
@@ -160,6 +176,27 @@ def main() -> int:
             drain()
         return sorted(times[1:])[1]  # median of the three after the warm-up run
 
+    if args.mixed:
+        lens = [rng.randrange(16, 2049) for _ in range(64)]
+        engine.scheduler.config = SchedulerConfig(
+            max_num_seqs=max_seqs, max_num_scheduled_tokens=PREFILL_TOKENS, max_num_partial_prefills=max_seqs,
+            max_long_partial_prefills=max_seqs, long_prefill_token_threshold=512)
+        for n in lens:
+            new_request(n, 128)
+        torch.cuda.synchronize()
+        t_start = time.perf_counter()
+        steps = 0
+        while engine.has_unfinished_requests():
+            engine.step()
+            steps += 1
+        torch.cuda.synchronize()
+        sec = time.perf_counter() - t_start
+        print(json.dumps({"workload": "mixed: 64 requests, prompts U[16,2048], portions of 512, 128 new tokens",
+                          "model": model_name, "dtype": args.dtype, "seconds": round(sec, 4), "steps": steps,
+                          "prompt_tokens": sum(lens), "generated_tokens": 64 * 128,
+                          "generated_tokens_per_s": round(64 * 128 / sec, 1),
+                          "total_tokens_per_s": round((sum(lens) + 64 * 128) / sec, 1)}))
+        return 0
     if args.only_prefill:
         sec = prefill_run()
         print(json.dumps({"prefill_tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3),
@@ -170,18 +207,18 @@ def main() -> int:
     bytes_step = weight_bytes_per_step(cfg, esize) + kv_bytes(cfg, args.batch, mean_ctx, esize)
     achieved = bytes_step / sec_per_step
     result = {
-        "metric": f"decode tok/s (Llama-3-8B shape, batch {args.batch}, 512-token prompts)",
+        "metric": f"decode tok/s ({model_name}, batch {args.batch}, {prompt_len}-token prompts)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {
-            "model": "llama-3-8b-shape-random", "layers": cfg["num_hidden_layers"],
+            "model": model_name, "layers": cfg["num_hidden_layers"],
             "layers_full": full_layers, "hidden": cfg["hidden_size"],
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"],
             "vocab": cfg["vocab_size"], "global_batch": args.batch, "seq_len": CONTEXT_LEN,
-            "prompt_len": PROMPT_LEN, "new_tokens": NEW_TOKENS, "page_size": PAGE_SIZE,
+            "prompt_len": prompt_len, "new_tokens": NEW_TOKENS, "page_size": PAGE_SIZE,
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single-gpu",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
