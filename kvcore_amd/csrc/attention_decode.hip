@@ -1,8 +1,11 @@
-// Paged attention for single tokens (decode), bfloat16, on the matrix cores.
+// Paged attention for single tokens (decode), bfloat16, on the matrix cores, with the
+// rotation of the token's query and key and the write of its key and value into the cache
+// done by the same kernel.
 //
-// One 64-lane wave per (token, kv head, split of the key range).  The query heads that
-// share the kv head are the columns of one 16-wide MFMA tile, so every key and value
-// is fetched once for the whole group, straight from global memory:
+// One block of W waves per (token, kv head, split of the key range); the waves take the
+// 16-key blocks of the range in turn.  The query heads that share the kv head are the
+// columns of one 16-wide MFMA tile, so every key and value is fetched once for the whole
+// group, straight from global memory:
 //
 //   S^T[16 keys, 16 heads]  = K[16 keys, d]       * Q^T[d, 16 heads]     (16x16x32)
 //   O^T[d, 16 heads]       += V^T[d, 16 keys]     * P^T[16 keys, 16 heads] (16x16x16)
@@ -13,9 +16,16 @@
 // probabilities never leave registers.  Softmax state (max, sum) is float32, one per
 // head, kept redundantly by the four lanes that hold a head's column.
 //
-// With more than one split each wave writes an unnormalised partial (max, sum,
-// output) and a second kernel combines them; split boundaries depend on the
-// request's length only.
+// The block first rotates the group's query heads into LDS.  The block whose range holds
+// the token's own position also rotates the key, stores key and value in their cache slot
+// and keeps both in LDS; the wave that meets the position's 16-key block takes them from
+// there, so nothing is read back from global memory in the kernel that wrote it.
+//
+// The waves' partial results (max, sum, output) are merged through LDS in wave order.
+// With more than one split each block writes an unnormalised partial and a second kernel
+// combines them; split boundaries depend on the request's length only.  (Letting the last
+// block to finish do that combination needs a device-wide fence per block, which costs
+// more than the second kernel.)
 
 #include <hip/hip_runtime.h>
 
@@ -31,64 +41,169 @@ typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kMaxWaves = 8;
+constexpr int kQPad = 8;    // bf16 elements between query rows in LDS beyond d
+constexpr int kOPad = 16;   // floats between output rows in LDS beyond d
+constexpr size_t kLdsLimit = 64 * 1024;
+
+struct DecodeArgs {
+  bf16_t* out;
+  float* part_o;
+  float* part_ml;
+  const bf16_t* qkv;  // rows [nh q heads | nkv k heads | nkv v heads] of d
+  int64_t qkv_stride;
+  bf16_t* k_cache;
+  bf16_t* v_cache;
+  const int32_t* table;
+  int table_stride;
+  const int32_t* positions;
+  const int32_t* token_req;
+  const int32_t* slots;
+  const float* cos_tab;  // [T, rot_dim / 2]
+  const float* sin_tab;
+  int rot_dim;
+  int interleaved;
+  int write_kv;  // store the token's key and value (and attend to them from LDS)
+  int nh, nkv, page_size, num_pages;
+  float scale_log2e;
+  int window;
+  int nsplit;
+};
+
+__host__ __device__ inline size_t lds_q_bytes(int g, int d) {
+  return (static_cast<size_t>(g) * (d + kQPad) * 2 + 15) / 16 * 16;
+}
+__host__ __device__ inline size_t lds_kv_bytes(int d) { return static_cast<size_t>(2) * d * 2; }
+__host__ __device__ inline size_t lds_ml_bytes(int waves) { return static_cast<size_t>(waves) * 16 * 8; }
+__host__ __device__ inline size_t lds_o_bytes(int waves, int g, int d) {
+  return static_cast<size_t>(waves) * g * (d + kOPad) * 4;
+}
+inline size_t lds_total(int waves, int g, int d) {
+  return lds_q_bytes(g, d) + lds_kv_bytes(d) + lds_ml_bytes(waves) + lds_o_bytes(waves, g, d);
+}
+
+// wide heads keep more registers per lane, so fewer waves fit in a block
+template <int D>
+constexpr int max_waves() { return D > 128 ? 4 : kMaxWaves; }
 
 template <int D>
-__global__ __launch_bounds__(64) void decode_attention_kernel(
-    bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
-    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_cache,
-    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ table, int table_stride,
-    const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
-    const int32_t* __restrict__ slots, int nh, int nkv, int page_size, int num_pages,
-    float scale_log2e, int window, int nsplit) {
+__global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(const DecodeArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int t = blockIdx.x;
   const int hk = blockIdx.y;
   const int split = blockIdx.z;
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x;
+  const int nthreads = blockDim.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int waves = nthreads >> 6;
+  const int lane = tid & 63;
   const int col = lane & 15;   // head within the group (B/C column)
   const int quad = lane >> 4;  // 0..3
+  const int nh = a.nh, nkv = a.nkv, nsplit = a.nsplit, page_size = a.page_size;
   const int g = nh / nkv;
   const int head = hk * g + col;
   const bool head_live = col < g;
-
-  const int req = token_req[t];
   constexpr int NJ = D / 16;  // output row blocks
   constexpr int NC = D / 32;  // 32-wide chunks of the head for Q.K
+
+  bf16_t* sq = reinterpret_cast<bf16_t*>(lds);                       // [g][D + kQPad]
+  bf16_t* sk = reinterpret_cast<bf16_t*>(lds + lds_q_bytes(g, D));   // [D] key, then [D] value
+  bf16_t* sv = sk + D;
+  float* sml = reinterpret_cast<float*>(lds + lds_q_bytes(g, D) + lds_kv_bytes(D));  // [waves][16][2]
+  float* so = sml + waves * 32;                                      // [waves][g][D + kOPad]
+
+  const int req = a.token_req[t];
   if (req < 0) {  // padding token
-    if (nsplit == 1 && head_live) {
-      bf16_t* o = out + (static_cast<int64_t>(t) * nh + head) * D;
-      for (int j = 0; j < NJ; ++j)
-        for (int i = 0; i < 4; ++i) o[16 * j + 4 * quad + i] = from_float<bf16_t>(0.f);
-    } else if (head_live && quad == 0) {
-      float* ml = part_ml + ((static_cast<int64_t>(t) * nh + head) * nsplit + split) * 2;
+    if (nsplit == 1) {
+      for (int idx = tid; idx < g * D; idx += nthreads)
+        a.out[(static_cast<int64_t>(t) * nh + hk * g) * D + idx] = from_float<bf16_t>(0.f);
+    } else if (tid < g) {
+      float* ml = a.part_ml + ((static_cast<int64_t>(t) * nh + hk * g + tid) * nsplit + split) * 2;
       ml[0] = -INFINITY;
       ml[1] = 0.f;
     }
     return;
   }
-  const int pos = positions[t];
+  const int pos = a.positions[t];
+  const int window = a.window;
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int32_t* row = table + static_cast<int64_t>(slots[req]) * table_stride;
+  const int32_t* row = a.table + static_cast<int64_t>(a.slots[req]) * a.table_stride;
 
-  // the 16-key blocks this wave owns: blocks [b0, b1) of the range that holds keys first..pos
+  // the 16-key blocks this block owns: [b0, b1) of the range that holds keys first..pos
   const int blk_first = first / 16;
   const int blk_end = pos / 16 + 1;
   const int nblk = blk_end - blk_first;
   const int per = (nblk + nsplit - 1) / nsplit;
   const int b0 = blk_first + split * per;
   const int b1 = (b0 + per < blk_end) ? b0 + per : blk_end;
+  const int blk_own = pos / 16;  // the block of the token's own key
+  const bool owner = a.write_kv && b0 <= blk_own && blk_own < b1;
+
+  // ---- rotation of the group's queries (and the key) into LDS; key and value into the cache
+  {
+    const bf16_t* trow = a.qkv + static_cast<int64_t>(t) * a.qkv_stride;
+    const int rot_dim = a.rot_dim, half = rot_dim / 2;
+    const float* cs = a.cos_tab + static_cast<int64_t>(t) * half;
+    const float* sn = a.sin_tab + static_cast<int64_t>(t) * half;
+    int64_t k_off = -1, v_off = -1;
+    if (owner) {
+      const int page = (pos / page_size < a.table_stride) ? row[pos / page_size] : 0;
+      if (page > 0 && page < a.num_pages) {
+        const int off = pos % page_size;
+        k_off = ((static_cast<int64_t>(page) * nkv + hk) * page_size + off) * D;
+        v_off = (static_cast<int64_t>(page) * nkv + hk) * D * page_size + off;
+      }
+    }
+    const int n_heads = owner ? g + 1 : g;  // the key is one more head to rotate
+    for (int idx = tid; idx < n_heads * D; idx += nthreads) {
+      const int hh = idx / D;
+      const int e = idx - hh * D;
+      const bf16_t* src = (hh < g) ? trow + static_cast<int64_t>(hk * g + hh) * D
+                                   : trow + static_cast<int64_t>(nh + hk) * D;
+      bf16_t y = src[e];
+      if (e < rot_dim) {
+        int j, partner;
+        bool is_first;
+        if (a.interleaved) {
+          j = e >> 1;
+          is_first = (e & 1) == 0;
+          partner = is_first ? e + 1 : e - 1;
+        } else {
+          is_first = e < half;
+          j = is_first ? e : e - half;
+          partner = is_first ? e + half : e - half;
+        }
+        const float c = cs[j], s_ = sn[j];
+        const float xe = to_float(y), xp = to_float(src[partner]);
+        y = from_float<bf16_t>(is_first ? rotate_first(xe, xp, c, s_) : rotate_second(xp, xe, c, s_));
+      }
+      if (hh < g) {
+        sq[hh * (D + kQPad) + e] = y;
+      } else {
+        sk[e] = y;
+        if (k_off >= 0) a.k_cache[k_off + e] = y;
+      }
+    }
+    if (owner) {
+      const bf16_t* vsrc = trow + static_cast<int64_t>(nh + nkv + hk) * D;
+      for (int e = tid; e < D; e += nthreads) {
+        const bf16_t v = vsrc[e];
+        sv[e] = v;
+        if (v_off >= 0) a.v_cache[v_off + static_cast<int64_t>(e) * page_size] = v;
+      }
+    }
+  }
+  __syncthreads();
 
   // Q^T as B operand: lane holds head `col`, elements 32c + 8*quad .. +8
   bf16x8_t bq[NC];
-  {
-    const bf16_t* qh = q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(head_live ? head : 0) * D;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      if (head_live) {
-        bq[c] = *reinterpret_cast<const bf16x8_t*>(qh + 32 * c + 8 * quad);
-      } else {
+  for (int c = 0; c < NC; ++c) {
+    if (head_live) {
+      bq[c] = *reinterpret_cast<const bf16x8_t*>(sq + col * (D + kQPad) + 32 * c + 8 * quad);
+    } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) bq[c][e] = static_cast<__bf16>(0.f);
-      }
+      for (int e = 0; e < 8; ++e) bq[c][e] = static_cast<__bf16>(0.f);
     }
   }
 
@@ -98,98 +213,151 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
   float m = -INFINITY, l = 0.f;
 
   const int blocks_per_page = page_size / 16;
-  for (int b = b0; b < b1; ++b) {
+  // one 16-key block: K rows as A operand (row = key `col`, elements 32c + 8*quad .. +8) and
+  // V^T rows (row = element 16j + col, keys 4*quad .. +4)
+  auto load_block = [&](int b, bf16x8_t (&ka)[NC], s16x4_t (&va)[NJ]) -> bool {
     const int page_idx = b / blocks_per_page;
     const int sub = b - page_idx * blocks_per_page;
-    const int page = row[page_idx];
-    if (page <= 0 || page >= num_pages) continue;  // a page given back behind the window
-    const bf16_t* kb = k_cache + ((static_cast<int64_t>(page) * nkv + hk) * page_size + sub * 16) * D;
-    const bf16_t* vb = v_cache + (static_cast<int64_t>(page) * nkv + hk) * D * page_size + sub * 16;
-
-    // S^T = K Q^T: A operand row = key `col`, elements 32c + 8*quad .. +8
-    f32x4_t s = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    const bf16_t* krow = kb + static_cast<int64_t>(col) * D + 8 * quad;
+    const int page = (page_idx < a.table_stride) ? row[page_idx] : 0;
+    if (page <= 0 || page >= a.num_pages) return false;  // a page given back behind the window
+    const bf16_t* krow = a.k_cache +
+                         ((static_cast<int64_t>(page) * nkv + hk) * page_size + sub * 16 + col) * D + 8 * quad;
+    const bf16_t* vrow = a.v_cache + ((static_cast<int64_t>(page) * nkv + hk) * D + col) * page_size +
+                         sub * 16 + 4 * quad;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(krow + 32 * c);
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[c], s, 0, 0, 0);
-    }
-    // V^T rows for the second product, fetched early: row = element 16j + col, keys 4*quad .. +4
-    s16x4_t va[NJ];
-    const bf16_t* vrow = vb + static_cast<int64_t>(col) * page_size + 4 * quad;
+    for (int c = 0; c < NC; ++c) ka[c] = *reinterpret_cast<const bf16x8_t*>(krow + 32 * c);
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
       va[j] = *reinterpret_cast<const s16x4_t*>(vrow + static_cast<int64_t>(16 * j) * page_size);
+    return true;
+  };
 
-    // s[i] belongs to key 16b + 4*quad + i and head `col`
-    const int key0 = 16 * b + 4 * quad;
-    float sv[4];
-    bool ok[4];
-    float mx = -INFINITY;
+  bf16x8_t k_cur[NC], k_next[NC];
+  s16x4_t v_cur[NJ], v_next[NJ];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = key0 + i;
-      ok[i] = key >= first && key <= pos;
-      sv[i] = ok[i] ? s[i] * scale_log2e : -INFINITY;
-      mx = fmaxf(mx, sv[i]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
-    float p[4];
-    float ps = 0.f;
+  for (int c = 0; c < NC; ++c) k_next[c] = bq[c];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      p[i] = __builtin_amdgcn_exp2f(sv[i] - m_safe);  // exp2(-inf) = 0 for masked keys
-      ps += p[i];
-    }
-    ps += __shfl_xor(ps, 16, 64);
-    ps += __shfl_xor(ps, 32, 64);
-    l = l * alpha + ps;
-    m = m_new;
-
-    // P^T as B operand of the 16x16x16 product: k = key 4*quad + i, column = head
-    s16x4_t pb;
+  for (int j = 0; j < NJ; ++j) v_next[j] = s16x4_t{0, 0, 0, 0};
+  bool ok_cur = false, ok_next = false;
+  int b = b0 + wave;
+  if (b < b1) ok_cur = load_block(b, k_cur, v_cur);
+  for (; b < b1; b += waves) {
+    const int bn = b + waves;
+    if (bn < b1) ok_next = load_block(bn, k_next, v_next);
+    if (ok_cur) {
+      if (owner && b == blk_own) {
+        // the token's own key and value come from LDS, not from the cache line just written
+        const int kk = pos & 15;
+        if (col == kk) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) pb[i] = static_cast<short>(f32_to_bf16_bits(p[i]));
-    // values of masked keys may be anything (a reused page, NaN): they must not meet the
-    // product even with weight zero
-    const bool edge = (16 * b + 15 > pos) || (16 * b < first);
+          for (int c = 0; c < NC; ++c)
+            k_cur[c] = *reinterpret_cast<const bf16x8_t*>(sk + 32 * c + 8 * quad);
+        }
+        if (quad == (kk >> 2)) {
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      s16x4_t a = va[j];
-      if (edge) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (!ok[i]) a[i] = 0;
+          for (int j = 0; j < NJ; ++j) {
+            const short bits = static_cast<short>(sv[16 * j + col].bits);
+            if ((kk & 3) == 0) v_cur[j][0] = bits;
+            if ((kk & 3) == 1) v_cur[j][1] = bits;
+            if ((kk & 3) == 2) v_cur[j][2] = bits;
+            if ((kk & 3) == 3) v_cur[j][3] = bits;
+          }
+        }
       }
-      o[j] = o[j] * alpha;
-      o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, o[j], 0, 0, 0);
+      f32x4_t s = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_cur[c], bq[c], s, 0, 0, 0);
+
+      // s[i] belongs to key 16b + 4*quad + i and head `col`
+      const int key0 = 16 * b + 4 * quad;
+      float sv4[4];
+      bool ok[4];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = key0 + i;
+        ok[i] = key >= first && key <= pos;
+        sv4[i] = ok[i] ? s[i] * a.scale_log2e : -INFINITY;
+        mx = fmaxf(mx, sv4[i]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m, mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+      float p[4];
+      float ps = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[i] = __builtin_amdgcn_exp2f(sv4[i] - m_safe);  // exp2(-inf) = 0 for masked keys
+        ps += p[i];
+      }
+      ps += __shfl_xor(ps, 16, 64);
+      ps += __shfl_xor(ps, 32, 64);
+      l = l * alpha + ps;
+      m = m_new;
+
+      // P^T as B operand of the 16x16x16 product: k = key 4*quad + i, column = head
+      s16x4_t pb;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pb[i] = static_cast<short>(f32_to_bf16_bits(p[i]));
+      // values of masked keys may be anything (a reused page, NaN): they must not meet the
+      // product even with weight zero
+      const bool edge = (16 * b + 15 > pos) || (16 * b < first);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        s16x4_t va = v_cur[j];
+        if (edge) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (!ok[i]) va[i] = 0;
+        }
+        o[j] = o[j] * alpha;
+        o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb, o[j], 0, 0, 0);
+      }
     }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) k_cur[c] = k_next[c];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) v_cur[j] = v_next[j];
+    ok_cur = ok_next;
   }
 
-  if (!head_live) return;
+  // ---- merge the waves' partials in wave order
   // o[j][i] = O^T[element 16j + 4*quad + i, head col]
-  if (nsplit == 1) {
-    const float inv = (l > 0.f) ? 1.f / l : 0.f;
-    bf16_t* op = out + (static_cast<int64_t>(t) * nh + head) * D + 4 * quad;
+  if (head_live) {
+    float* wo = so + (static_cast<int64_t>(wave) * g + col) * (D + kOPad) + 4 * quad;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      uint2 packed;
-      packed.x = f32_to_bf16_bits(o[j][0] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[j][1] * inv)) << 16);
-      packed.y = f32_to_bf16_bits(o[j][2] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[j][3] * inv)) << 16);
-      *reinterpret_cast<uint2*>(op + 16 * j) = packed;
-    }
-  } else {
-    const int64_t slot_idx = (static_cast<int64_t>(t) * nh + head) * nsplit + split;
-    float* po = part_o + slot_idx * D + 4 * quad;
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) *reinterpret_cast<f32x4_t*>(po + 16 * j) = o[j];
+    for (int j = 0; j < NJ; ++j) *reinterpret_cast<f32x4_t*>(wo + 16 * j) = o[j];
     if (quad == 0) {
-      part_ml[slot_idx * 2] = m;
-      part_ml[slot_idx * 2 + 1] = l;
+      sml[(wave * 16 + col) * 2] = m;
+      sml[(wave * 16 + col) * 2 + 1] = l;
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < g * D; idx += nthreads) {
+    const int h = idx / D;
+    const int e = idx - h * D;
+    float mmax = -INFINITY;
+    for (int w = 0; w < waves; ++w) mmax = fmaxf(mmax, sml[(w * 16 + h) * 2]);
+    const float m_safe = (mmax == -INFINITY) ? 0.f : mmax;
+    float denom = 0.f, acc = 0.f;
+    for (int w = 0; w < waves; ++w) {
+      const float wgt = __builtin_amdgcn_exp2f(sml[(w * 16 + h) * 2] - m_safe);
+      if (wgt > 0.f) {
+        denom += wgt * sml[(w * 16 + h) * 2 + 1];
+        acc += wgt * so[(static_cast<int64_t>(w) * g + h) * (D + kOPad) + e];
+      }
+    }
+    const int64_t th = static_cast<int64_t>(t) * nh + hk * g + h;
+    if (nsplit == 1) {
+      a.out[th * D + e] = from_float<bf16_t>(denom > 0.f ? acc / denom : 0.f);
+    } else {
+      a.part_o[(th * nsplit + split) * D + e] = acc;
+      if (e == 0) {
+        a.part_ml[(th * nsplit + split) * 2] = mmax;
+        a.part_ml[(th * nsplit + split) * 2 + 1] = denom;
+      }
     }
   }
 }
@@ -197,36 +365,53 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
 // out[t, head, :] = sum_s w_s * part_o[s] / sum_s w_s * l_s with w_s = exp2(m_s - max m)
 __global__ void decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                                       const float* __restrict__ part_ml, int D, int nsplit) {
+  extern __shared__ float wgt[];  // [nsplit]
+  __shared__ float inv_denom;
   const int64_t th = blockIdx.x;  // token * nh + head
   const float* ml = part_ml + th * nsplit * 2;
-  float mmax = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) mmax = fmaxf(mmax, ml[2 * s]);
-  const float m_safe = (mmax == -INFINITY) ? 0.f : mmax;
-  float denom = 0.f;
-  for (int s = 0; s < nsplit; ++s) denom += __builtin_amdgcn_exp2f(ml[2 * s] - m_safe) * ml[2 * s + 1];
-  const float inv = (denom > 0.f) ? 1.f / denom : 0.f;
+  if (threadIdx.x < 64) {  // the first wave: weights of the splits
+    float mmax = -INFINITY;
+    for (int s = threadIdx.x; s < nsplit; s += 64) mmax = fmaxf(mmax, ml[2 * s]);
+    mmax = wave_max(mmax);
+    const float m_safe = (mmax == -INFINITY) ? 0.f : mmax;
+    for (int s = threadIdx.x; s < nsplit; s += 64) wgt[s] = __builtin_amdgcn_exp2f(ml[2 * s] - m_safe);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float denom = 0.f;
+    for (int s = 0; s < nsplit; ++s) denom += wgt[s] * ml[2 * s + 1];
+    inv_denom = (denom > 0.f) ? 1.f / denom : 0.f;
+  }
+  __syncthreads();
+  const float inv = inv_denom;
   for (int e = threadIdx.x; e < D; e += blockDim.x) {
     float acc = 0.f;
     for (int s = 0; s < nsplit; ++s) {
-      const float w = __builtin_amdgcn_exp2f(ml[2 * s] - m_safe);
+      const float w = wgt[s];
       if (w > 0.f) acc += w * part_o[(th * nsplit + s) * D + e];
     }
     out[th * D + e] = from_float<bf16_t>(acc * inv);
   }
 }
 
+int decode_waves(int g, int d) {
+  int waves = d > 128 ? 4 : kMaxWaves;
+  while (waves > 1 && lds_total(waves, g, d) > kLdsLimit) waves /= 2;
+  return waves;
+}
+
 template <int D>
-int launch_decode(bf16_t* out, float* part_o, float* part_ml, const bf16_t* q, int64_t q_stride,
-                  const bf16_t* k_cache, const bf16_t* v_cache, const int32_t* table,
-                  int table_stride, const int32_t* positions, const int32_t* token_req,
-                  const int32_t* slots, int T, int nh, int nkv, int page_size, int num_pages,
-                  float scale, int window, int nsplit, hipStream_t stream) {
-  hipLaunchKernelGGL(decode_attention_kernel<D>, dim3(T, nkv, nsplit), dim3(64), 0, stream, out,
-                     part_o, part_ml, q, q_stride, k_cache, v_cache, table, table_stride, positions,
-                     token_req, slots, nh, nkv, page_size, num_pages, scale * kLog2e, window, nsplit);
-  if (nsplit > 1)
-    hipLaunchKernelGGL(decode_combine_kernel, dim3(T * nh), dim3(D < 64 ? 64 : D), 0, stream, out,
-                       part_o, part_ml, D, nsplit);
+int launch_decode(const DecodeArgs& args, int T, hipStream_t stream) {
+  const int g = args.nh / args.nkv;
+  int waves = decode_waves(g, D);
+  // more blocks than compute units: smaller blocks pack better
+  if (static_cast<int64_t>(T) * args.nkv * args.nsplit > 256 && waves > 4) waves = 4;
+  hipLaunchKernelGGL(decode_attention_kernel<D>, dim3(T, args.nkv, args.nsplit), dim3(waves * 64),
+                     lds_total(waves, g, D), stream, args);
+  if (args.nsplit > 1)
+    hipLaunchKernelGGL(decode_combine_kernel, dim3(T * args.nh), dim3(D < 64 ? 64 : D),
+                       args.nsplit * sizeof(float), stream, args.out, args.part_o, args.part_ml, D,
+                       args.nsplit);
   return kvc_check_launch("kvc_decode_attention");
 }
 
@@ -239,41 +424,68 @@ extern "C" int kvc_decode_attention_supported(int nh, int nkv, int d, int page_s
   return d == 32 || d == 64 || d == 96 || d == 128 || d == 160 || d == 192 || d == 224 || d == 256;
 }
 
-extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* q,
-                                    int64_t q_stride, const void* k_cache, const void* v_cache,
+extern "C" int kvc_decode_attention_waves(int nh, int nkv, int d) {
+  if (nkv <= 0 || nh % nkv || d <= 0) return 0;
+  return decode_waves(nh / nkv, d);
+}
+
+extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* qkv,
+                                    int64_t qkv_stride, void* k_cache, void* v_cache,
                                     const int32_t* table, int table_stride,
                                     const int32_t* positions, const int32_t* token_req,
-                                    const int32_t* slots, int T, int nh, int nkv, int d,
-                                    int page_size, int num_pages, float scale, int window,
-                                    int nsplit, kvc_stream stream) {
+                                    const int32_t* slots, const float* cos_tab, const float* sin_tab,
+                                    int rot_dim, int interleaved, int write_kv, int T, int nh,
+                                    int nkv, int d, int page_size, int num_pages, float scale,
+                                    int window, int nsplit, kvc_stream stream) {
   if (!kvc_decode_attention_supported(nh, nkv, d, page_size, 1))
     return kvc_fail("kvc_decode_attention: unsupported shape (bfloat16, head size a multiple of 32 "
                     "up to 256, at most 16 query heads per kv head, page size a multiple of 16)");
   if (T < 0 || nsplit < 1 || nsplit > 65535 || nkv > 65535 || table_stride <= 0 || num_pages <= 0)
     return kvc_fail("kvc_decode_attention: bad sizes");
-  if (q_stride % 8) return kvc_fail("kvc_decode_attention: q rows must be 16-byte aligned");
+  if (qkv_stride % 8 || qkv_stride < static_cast<int64_t>(nh + (write_kv ? 2 * nkv : 0)) * d)
+    return kvc_fail("kvc_decode_attention: token rows must be 16-byte aligned and hold q (and k, v)");
+  if (rot_dim < 0 || rot_dim > d || rot_dim % 2)
+    return kvc_fail("kvc_decode_attention: the rotated width must be even and at most the head size");
+  if (rot_dim > 0 && (cos_tab == nullptr || sin_tab == nullptr))
+    return kvc_fail("kvc_decode_attention: rotation needs its cos and sin tables");
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr))
     return kvc_fail("kvc_decode_attention: splits need a workspace");
   if (T == 0) return 0;
+  DecodeArgs args;
+  args.out = static_cast<bf16_t*>(out);
+  args.part_o = static_cast<float*>(part_o);
+  args.part_ml = static_cast<float*>(part_ml);
+  args.qkv = static_cast<const bf16_t*>(qkv);
+  args.qkv_stride = qkv_stride;
+  args.k_cache = static_cast<bf16_t*>(k_cache);
+  args.v_cache = static_cast<bf16_t*>(v_cache);
+  args.table = table;
+  args.table_stride = table_stride;
+  args.positions = positions;
+  args.token_req = token_req;
+  args.slots = slots;
+  args.cos_tab = cos_tab;
+  args.sin_tab = sin_tab;
+  args.rot_dim = rot_dim;
+  args.interleaved = interleaved;
+  args.write_kv = write_kv;
+  args.nh = nh;
+  args.nkv = nkv;
+  args.page_size = page_size;
+  args.num_pages = num_pages;
+  args.scale_log2e = scale * kLog2e;
+  args.window = window;
+  args.nsplit = nsplit;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-#define KVC_DECODE_CASE(DD)                                                                       \
-  case DD:                                                                                        \
-    return launch_decode<DD>(static_cast<bf16_t*>(out), static_cast<float*>(part_o),              \
-                             static_cast<float*>(part_ml), static_cast<const bf16_t*>(q),         \
-                             q_stride, static_cast<const bf16_t*>(k_cache),                       \
-                             static_cast<const bf16_t*>(v_cache), table, table_stride, positions, \
-                             token_req, slots, T, nh, nkv, page_size, num_pages, scale, window,   \
-                             nsplit, s)
   switch (d) {
-    KVC_DECODE_CASE(32);
-    KVC_DECODE_CASE(64);
-    KVC_DECODE_CASE(96);
-    KVC_DECODE_CASE(128);
-    KVC_DECODE_CASE(160);
-    KVC_DECODE_CASE(192);
-    KVC_DECODE_CASE(224);
-    KVC_DECODE_CASE(256);
+    case 32: return launch_decode<32>(args, T, s);
+    case 64: return launch_decode<64>(args, T, s);
+    case 96: return launch_decode<96>(args, T, s);
+    case 128: return launch_decode<128>(args, T, s);
+    case 160: return launch_decode<160>(args, T, s);
+    case 192: return launch_decode<192>(args, T, s);
+    case 224: return launch_decode<224>(args, T, s);
+    case 256: return launch_decode<256>(args, T, s);
   }
-#undef KVC_DECODE_CASE
   return kvc_fail("kvc_decode_attention: unsupported head size");
 }

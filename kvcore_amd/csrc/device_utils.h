@@ -38,6 +38,16 @@ __device__ __forceinline__ bf16_t from_float<bf16_t>(float x) {
   return r;
 }
 
+// One rotary pair (x0, x1) turned by the angle whose cosine and sine are c and s:
+// (x0 c - x1 s, x1 c + x0 s), each as one product and one fused multiply-add, so that every
+// kernel that rotates gives the same bits.
+__device__ __forceinline__ float rotate_first(float x0, float x1, float c, float s) {
+  return __builtin_fmaf(-x1, s, x0 * c);
+}
+__device__ __forceinline__ float rotate_second(float x0, float x1, float c, float s) {
+  return __builtin_fmaf(x0, s, x1 * c);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

@@ -457,8 +457,8 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
       load8(sn + j, s_);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        y0[e] = x0[e] * c[e] - x1[e] * s_[e];
-        y1[e] = x1[e] * c[e] + x0[e] * s_[e];
+        y0[e] = rotate_first(x0[e], x1[e], c[e], s_[e]);
+        y1[e] = rotate_second(x0[e], x1[e], c[e], s_[e]);
       }
       store8(hp + j, y0);
       store8(hp + j + half, y1);
@@ -479,8 +479,8 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
       const float x0 = to_float(hp[i0]);
       const float x1 = to_float(hp[i1]);
       const float c = cs[j], s_ = sn[j];
-      const T y0 = from_float<T>(x0 * c - x1 * s_);
-      const T y1 = from_float<T>(x1 * c + x0 * s_);
+      const T y0 = from_float<T>(rotate_first(x0, x1, c, s_));
+      const T y1 = from_float<T>(rotate_second(x0, x1, c, s_));
       hp[i0] = y0;
       hp[i1] = y1;
       if (head >= nh && k_base >= 0) {

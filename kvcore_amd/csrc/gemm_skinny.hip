@@ -56,25 +56,30 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v, int n_left)
   }
 }
 
-template <int RT, int NT, int U, int MAXW, typename OutT>
+// GATED: the two row tiles of a wave are rows n of the first N weight rows (gate) and rows
+// N + n (up), and the stored value is silu(gate) * up, each factor rounded to bfloat16
+// first as if it had been stored.
+template <int RT, int NT, int U, int MAXW, typename OutT, bool GATED>
 __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restrict__ A,
                                    const bf16_t* __restrict__ W, const bf16_t* __restrict__ bias,
                                    int M, int N, int K, int64_t lda, int64_t ldc, int k_per_wave) {
+  static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
   extern __shared__ float red[];  // [waves - 1][RT * NT][64][4]
   const int wave = threadIdx.x >> 6;
   const int waves = blockDim.x >> 6;
   const int lane = threadIdx.x & 63;
   const int col = lane & 15;
   const int quad = lane >> 4;
-  const int n0 = blockIdx.x * (16 * RT);
+  const int n0 = blockIdx.x * (GATED ? 16 : 16 * RT);
   const int k_begin = wave * k_per_wave;
   const int k_end = (k_begin + k_per_wave < K) ? k_begin + k_per_wave : K;
 
   const bf16_t* wp[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int r = n0 + rt * 16 + col;
-    wp[rt] = W + static_cast<int64_t>(r < N ? r : N - 1) * K + 8 * quad;
+    const int r = GATED ? n0 + col : n0 + rt * 16 + col;
+    const int64_t row = (r < N ? r : N - 1) + ((GATED && rt == 1) ? N : 0);
+    wp[rt] = W + row * K + 8 * quad;
   }
   const bf16_t* ap[NT];
   bool tok_ok[NT];
@@ -183,6 +188,31 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
   }
   // acc[rt][nt][i] = C[token nt*16 + col][n0 + rt*16 + 4*quad + i]; columns of unused tokens
   // multiplied whatever row 0 of A holds and are dropped here
+  if constexpr (GATED) {
+    const int n_first = n0 + 4 * quad;
+    const int n_left = N - n_first;
+    if (n_left <= 0) return;
+    f32x4_t bg = f32x4_t{0.f, 0.f, 0.f, 0.f}, bu = bg;
+    if (bias != nullptr)
+      for (int i = 0; i < 4 && i < n_left; ++i) {
+        bg[i] = to_float(bias[n_first + i]);
+        bu[i] = to_float(bias[N + n_first + i]);
+      }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int tok = nt * 16 + col;
+      if (tok >= M) continue;
+      f32x4_t y;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float gv = to_float(from_float<bf16_t>(acc[0][nt][i] + bg[i]));
+        const float uv = to_float(from_float<bf16_t>(acc[1][nt][i] + bu[i]));
+        y[i] = gv / (1.f + expf(-gv)) * uv;
+      }
+      store4<OutT>(C + static_cast<int64_t>(tok) * ldc + n_first, y, n_left);
+    }
+    return;
+  }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const int n_first = n0 + rt * 16 + 4 * quad;
@@ -200,16 +230,17 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
   }
 }
 
-template <int RT, int NT, typename OutT>
+template <int RT, int NT, typename OutT, bool GATED = false>
 void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
             int64_t lda, int64_t ldc, int waves, int k_per_wave, hipStream_t stream) {
   // steps in flight by what fits in registers beside the accumulators
   constexpr int STAGES = (RT + NT <= 5) ? 4 : ((RT + NT <= 6) ? 3 : 2);
   constexpr int MAXW = (RT >= 2) ? 4 : 8;
   const size_t lds = static_cast<size_t>(waves - 1) * RT * NT * 64 * 4 * sizeof(float);
-  hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, STAGES, MAXW, OutT>),
-                     dim3((N + 16 * RT - 1) / (16 * RT)), dim3(waves * 64), lds, stream, C, A, W,
-                     bias, M, N, K, lda, ldc, k_per_wave);
+  const int rows_per_block = GATED ? 16 : 16 * RT;
+  hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, STAGES, MAXW, OutT, GATED>),
+                     dim3((N + rows_per_block - 1) / rows_per_block), dim3(waves * 64), lds, stream,
+                     C, A, W, bias, M, N, K, lda, ldc, k_per_wave);
 }
 
 // The launch shape is a function of N and K alone, so that a row's sums do not depend on
@@ -259,7 +290,42 @@ int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int 
   return kvc_check_launch("kvc_gemm_skinny_bf16");
 }
 
+// silu(A Wg^T) * (A Wu^T) with Wg the first N rows of W and Wu the next N
+int dispatch_gated(bf16_t* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N,
+                   int K, int64_t lda, int64_t ldc, hipStream_t stream) {
+  int waves = 4;
+  while (waves > 1 && K / waves < 128) waves /= 2;
+  const int nt = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
+  int k_per_wave = (K + waves - 1) / waves;
+  k_per_wave = (k_per_wave + 63) / 64 * 64;
+#define KVC_SKINNY_GATED(NT_) \
+  launch<2, NT_, bf16_t, true>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream)
+  switch (nt) {
+    case 1: KVC_SKINNY_GATED(1); break;
+    case 2: KVC_SKINNY_GATED(2); break;
+    case 4: KVC_SKINNY_GATED(4); break;
+    default: return kvc_fail("kvc_gemm_skinny_silu_mul_bf16: unsupported launch shape");
+  }
+#undef KVC_SKINNY_GATED
+  return kvc_check_launch("kvc_gemm_skinny_silu_mul_bf16");
+}
+
 }  // namespace
+
+extern "C" int kvc_gemm_skinny_silu_mul_bf16(void* C, const void* A, const void* W, const void* bias,
+                                             int M, int N, int K, int64_t lda, int64_t ldc,
+                                             kvc_stream stream) {
+  if (M < 0 || M > 64 || N <= 0 || K <= 0 || lda < K || ldc < N)
+    return kvc_fail("kvc_gemm_skinny_silu_mul_bf16: bad sizes (1 to 64 rows)");
+  if (K % 8 || lda % 8)
+    return kvc_fail("kvc_gemm_skinny_silu_mul_bf16: K and the row stride must be multiples of 8");
+  if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15))
+    return kvc_fail("kvc_gemm_skinny_silu_mul_bf16: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  return dispatch_gated(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
+                        static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N, K,
+                        lda, ldc, reinterpret_cast<hipStream_t>(stream));
+}
 
 extern "C" int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M,
                                     int N, int K, int64_t lda, int64_t ldc, int out_dtype,

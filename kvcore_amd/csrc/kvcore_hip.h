@@ -75,19 +75,27 @@ int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* 
                         const int32_t* slots, int T, int nh, int nkv, int d, int page_size,
                         int num_pages, float scale, int window, int dtype, kvc_stream stream);
 
-// The same attention for bfloat16 on the matrix cores, one wave per (token, kv head,
-// split): meant for steps of single tokens.  nsplit > 1 needs part_o [T, nh, nsplit, d]
-// and part_ml [T, nh, nsplit, 2] float32; a second kernel combines the splits (a "last
-// wave combines" scheme needs device-scope fences, which on this chip write back and
-// invalidate a whole L2 slice per wave and cost more than the launch they save).
+// The same attention for bfloat16 steps of single tokens on the matrix cores, a block of
+// several waves per (token, kv head, split), which also does what kvc_rope_kv_write does for
+// its token: qkv rows are [nh q heads | nkv k heads | nkv v heads]; the first rot_dim elements
+// of every q head (and of the k head) are rotated by cos/sin [T, rot_dim / 2] on the way in
+// (rot_dim 0: taken as they are) and qkv itself is left unchanged; with write_kv the
+// token's key and value are stored in their cache slot and attended to (without write_kv
+// the cache must already hold them).  nsplit > 1 needs part_o [T, nh, nsplit, d] and part_ml
+// [T, nh, nsplit, 2] float32; a second kernel combines the splits (a "last block combines"
+// scheme needs device-scope fences, which on this chip write back and invalidate a whole L2
+// slice per block and cost more than the launch they save).
 // kvc_decode_attention_supported tells whether a shape is served (else use
-// kvc_paged_attention).
+// kvc_paged_attention); kvc_decode_attention_waves how many waves share a block's key range.
 int kvc_decode_attention_supported(int nh, int nkv, int d, int page_size, int dtype);
-int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* q, int64_t q_stride,
-                         const void* k_cache, const void* v_cache, const int32_t* table,
+int kvc_decode_attention_waves(int nh, int nkv, int d);
+int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* qkv,
+                         int64_t qkv_stride, void* k_cache, void* v_cache, const int32_t* table,
                          int table_stride, const int32_t* positions, const int32_t* token_req,
-                         const int32_t* slots, int T, int nh, int nkv, int d, int page_size,
-                         int num_pages, float scale, int window, int nsplit, kvc_stream stream);
+                         const int32_t* slots, const float* cos_tab, const float* sin_tab,
+                         int rot_dim, int interleaved, int write_kv, int T, int nh, int nkv, int d,
+                         int page_size, int num_pages, float scale, int window, int nsplit,
+                         kvc_stream stream);
 
 // The same attention for bfloat16 portions of prompts on the matrix cores: a block per
 // (tile of a request's tokens, kv head), keys staged through LDS.  q_start [R+1] bounds
@@ -110,6 +118,13 @@ int kvc_gemm_f32(float* C, const float* A, const float* W, const float* bias, in
 // K and lda must be multiples of 8, A and W 16-byte aligned.
 int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
                          int K, int64_t lda, int64_t ldc, int out_dtype, kvc_stream stream);
+
+// C[M, N] = silu(A Wg^T + bg) * (A Wu^T + bu) for M <= 64 rows of bfloat16, where Wg is rows
+// 0..N-1 of W[2N, K] and Wu rows N..2N-1 (bias[2N] likewise): the gated feed-forward's first
+// product with its activation, both factors rounded to bfloat16 before the activation as the
+// two-kernel form stores them.  C is bfloat16.
+int kvc_gemm_skinny_silu_mul_bf16(void* C, const void* A, const void* W, const void* bias, int M,
+                                  int N, int K, int64_t lda, int64_t ldc, kvc_stream stream);
 
 // table[triples[3i], triples[3i+1]] = triples[3i+2] for i < n.
 int kvc_table_update(int32_t* table, int table_stride, int table_rows, const int32_t* triples,

@@ -159,8 +159,8 @@ class ModelRunner:
         # steps of single tokens are captured once per batch-size bucket and replayed
         self.use_hip_graphs = use_hip_graphs and model.graph_safe()
         self._graph_buckets = _decode_buckets(min(max_num_seqs, max_num_tokens))
-        self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
-        self._graph_warm: set[int] = set()
+        self._graphs: dict[tuple[int, int], tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        self._graph_warm: set[tuple[int, int]] = set()
         self.graph_replays = 0
 
     def _drop_graphs(self) -> None:
@@ -346,7 +346,7 @@ class ModelRunner:
 
         ids = [e.request_id for e in entries]
         if bucket:
-            return StepOutput(ids, self._run_decode_bucket(bucket, R), owners, T)
+            return StepOutput(ids, self._run_decode_bucket(bucket, R, max(seq_lens)), owners, T)
         ctx = self._context(T, R, q_lens, seq_lens, max(q_lens), max(seq_lens))
         hidden = self.model.forward(ctx)
         logits = None
@@ -367,26 +367,32 @@ class ModelRunner:
             max_query_len=max_q, max_seq_len=max_seq,
         )
 
-    def _run_decode_bucket(self, bucket: int, num_live: int) -> torch.Tensor:
+    def _run_decode_bucket(self, bucket: int, num_live: int, max_seq_len: int) -> torch.Tensor:
         """A padded step of ``bucket`` single tokens.  The first such step runs launch by
         launch (which also sizes every step buffer); the second is captured into a HIP
         graph; from then on the graph is replayed.  Nothing in the graph depends on the
         batch beyond what the index arrays on the device say: the context it was captured
-        with claims the longest sequence the engine allows."""
+        with claims a sequence length that bounds the batch's (the next power of two, at
+        least 1024, at most the engine's limit), so that the parts may plan their launches
+        by it; each such length class has a graph of its own."""
+        plan_len = 1024
+        while plan_len < max_seq_len:
+            plan_len *= 2
+        plan_len = min(plan_len, self.max_model_len)
+        key = (bucket, plan_len)
 
         def run() -> torch.Tensor:
-            ctx = self._context(bucket, bucket, [1] * bucket, [self.max_model_len] * bucket, 1,
-                                self.max_model_len)
+            ctx = self._context(bucket, bucket, [1] * bucket, [plan_len] * bucket, 1, plan_len)
             hidden = self.model.forward(ctx)
             return self.model.compute_logits(ctx, hidden, self._dev["logit_rows"], bucket)
 
-        if bucket in self._graphs:
-            graph, logits = self._graphs[bucket]
+        if key in self._graphs:
+            graph, logits = self._graphs[key]
             graph.replay()
             self.graph_replays += 1
             return logits[:num_live]
-        if bucket not in self._graph_warm:
-            self._graph_warm.add(bucket)
+        if key not in self._graph_warm:
+            self._graph_warm.add(key)
             return run()[:num_live]
         graph = torch.cuda.CUDAGraph()
         self.buffers.frozen = True
@@ -403,7 +409,7 @@ class ModelRunner:
             if gc_was_enabled:
                 gc.enable()
             self.buffers.frozen = False
-        self._graphs[bucket] = (graph, logits)
+        self._graphs[key] = (graph, logits)
         graph.replay()
         self.graph_replays += 1
         return logits[:num_live]

@@ -40,12 +40,15 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
         "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, P],
         "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
-        "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
+                                 F, I, I, P],
+        "kvc_decode_attention_waves": [I, I, I],
         "kvc_decode_attention_supported": [I, I, I, I, I],
         "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kvc_prefill_attention_supported": [I, I, I, I, I],
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
         "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, P],
+        "kvc_gemm_skinny_silu_mul_bf16": [P, P, P, P, I, I, I, L, L, P],
         "kvc_table_update": [P, I, I, P, I, P],
         "kvc_argmax": [P, P, I, I, L, P, P, I, P],
         "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P],
@@ -253,24 +256,41 @@ def decode_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype:
     return bool(load().kvc_decode_attention_supported(nh, nkv, d, page_size, DTYPE_CODE.get(dtype, -1)))
 
 
-def decode_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+def decode_attention_waves(nh: int, nkv: int, d: int) -> int:
+    """How many waves of a block share its range of keys in :func:`decode_attention`."""
+    return int(load().kvc_decode_attention_waves(nh, nkv, d))
+
+
+def decode_attention(out: torch.Tensor, qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      *, table: torch.Tensor, positions: torch.Tensor, token_req: torch.Tensor,
                      slots: torch.Tensor, nh: int, nkv: int, d: int, scale: float, window: int = 0,
                      nsplit: int = 1, part_o: torch.Tensor | None = None,
-                     part_ml: torch.Tensor | None = None) -> None:
-    """bfloat16 attention of single tokens on the matrix cores (see the C header).  ``part_o``
-    and ``part_ml`` are float32 workspaces of at least ``T*nh*nsplit*d`` and ``T*nh*nsplit*2``
+                     part_ml: torch.Tensor | None = None, cos: torch.Tensor | None = None,
+                     sin: torch.Tensor | None = None, rot_dim: int = 0, interleaved: bool = False,
+                     write_kv: bool = False) -> None:
+    """bfloat16 attention of single tokens on the matrix cores (see the C header), with the
+    rotation of each token's query and key and the write of its key and value into the cache
+    (``write_kv``) in the same kernel; ``qkv`` is not changed.  With ``rot_dim = 0`` and
+    ``write_kv = False`` it is the attention alone over queries as they are.  ``part_o`` and
+    ``part_ml`` are float32 workspaces of at least ``T*nh*nsplit*d`` and ``T*nh*nsplit*2``
     elements when ``nsplit > 1``."""
     T = out.shape[0]
     if out.shape != (T, nh * d) or not out.is_contiguous() or out.dtype != torch.bfloat16:
         raise KernelError("decode_attention: out must be contiguous bfloat16 [T, nh*d]")
-    if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or q.dtype != out.dtype:
-        raise KernelError("decode_attention: q does not fit")
+    need = (nh + 2 * nkv) * d if write_kv else nh * d
+    if qkv.shape[0] != T or qkv.stride(1) != 1 or qkv.shape[1] < need or qkv.dtype != out.dtype:
+        raise KernelError("decode_attention: qkv does not fit")
     num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "decode_attention")
     if k_cache.dtype != out.dtype:
         raise KernelError("decode_attention: cache dtype differs from the queries'")
     if positions.numel() < T or token_req.numel() < T:
         raise KernelError("decode_attention: per-token arrays too short")
+    c = s_ = None
+    if rot_dim:
+        if cos is None or sin is None or cos.shape[0] < T or cos.shape[1] != rot_dim // 2 \
+                or sin.shape != cos.shape or not cos.is_contiguous() or not sin.is_contiguous():
+            raise KernelError("decode_attention: cos and sin must be contiguous [>= T, rot_dim/2]")
+        c, s_ = _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32)
     po = pm = None
     if nsplit > 1:
         if part_o is None or part_ml is None or part_o.numel() < T * nh * nsplit * d \
@@ -278,10 +298,11 @@ def decode_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
             raise KernelError("decode_attention: workspace missing or too small")
         po, pm = _dev(part_o, "part_o", torch.float32), _dev(part_ml, "part_ml", torch.float32)
     _check(load().kvc_decode_attention(
-        out.data_ptr(), po, pm, q.data_ptr(), q.stride(0), _dev(k_cache, "k_cache"),
+        out.data_ptr(), po, pm, qkv.data_ptr(), qkv.stride(0), _dev(k_cache, "k_cache"),
         _dev(v_cache, "v_cache"), _dev(table, "table", torch.int32), table.shape[1],
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
-        _dev(slots, "slots", torch.int32), T, nh, nkv, d, page_size, num_pages, float(scale),
+        _dev(slots, "slots", torch.int32), c, s_, int(rot_dim), int(bool(interleaved)),
+        int(bool(write_kv)), T, nh, nkv, d, page_size, num_pages, float(scale),
         int(window), int(nsplit), _stream()), "kvc_decode_attention")
 
 
@@ -360,6 +381,36 @@ def gemm_skinny_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor,
            "kvc_gemm_skinny_bf16")
 
 
+def _skinny_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def linear_silu_mul(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None,
+                    scratch) -> None:
+    """``out = silu(x @ wg.T) * (x @ wu.T)`` with ``wg`` the first half of ``w``'s rows and
+    ``wu`` the second (biases likewise).  Few rows of bfloat16 run as one weight-streaming
+    kernel; otherwise ``scratch()`` gives the ``[M, 2I]`` buffer for the two-kernel form."""
+    M, K = x.shape
+    I = w.shape[0] // 2
+    if w.shape != (2 * I, K) or out.shape != (M, I):
+        raise KernelError("linear_silu_mul: shapes do not match")
+    if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+            and x.is_cuda and _skinny_operands_ok(x, w)
+            and (M <= 8 or (M <= SKINNY_PREFERRED_ROWS and K <= 8192))):
+        if M == 0:
+            return
+        if bias is not None and (bias.dtype != torch.bfloat16 or bias.shape != (2 * I,)):
+            raise KernelError("linear_silu_mul: bias must be bfloat16 [2I]")
+        _check(load().kvc_gemm_skinny_silu_mul_bf16(
+            out.data_ptr(), x.data_ptr(), _dev(w, "w"), None if bias is None else _dev(bias, "bias"),
+            M, I, K, x.stride(0), out.stride(0), _stream()), "kvc_gemm_skinny_silu_mul_bf16")
+        return
+    gate_up = scratch()
+    linear(gate_up, x, w, bias)
+    silu_mul(out, gate_up)
+
+
 def linear(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -> None:
     """``out = x @ w.T (+ bias)``.  float32 runs the library's own true-float32 kernel.
     bfloat16 with at most 64 rows runs the weight-streaming matrix-core kernel (float32
@@ -374,8 +425,7 @@ def linear(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tens
         return
     M, K = x.shape
     N = w.shape[0]
-    skinny_ok = (M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0
-                 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+    skinny_ok = _skinny_operands_ok(x, w)
     # measured on MI355X (N x K of 4096..128256 x 4096..14336): the weight-streaming kernel
     # wins up to 8 rows everywhere and up to 16 rows unless K or N is very large; it is also
     # the only one that stores float32

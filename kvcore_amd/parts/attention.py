@@ -15,16 +15,21 @@ from kvcore_amd.ops import library as ops
 from .base import CacheNeed, Mixer, ParamSource, ParamSpec, PositionEncoding, register_mixer
 
 
-DECODE_TARGET_WAVES = 1024  # enough single-wave blocks to keep 256 compute units fed
+DECODE_TARGET_WAVES = 1024  # enough waves to keep 256 compute units fed
 DECODE_MAX_SPLITS = 32
+DECODE_BLOCKS_PER_WAVE = 8  # 16-key blocks one wave may walk before the range is split
 
 
-def decode_splits(num_tokens: int, num_kv_heads: int, max_seq_len: int) -> int:
-    """Into how many parts each request's key range is cut for the decode kernel: enough
-    that tokens x kv heads x parts fills the chip, never more than there are 16-key blocks."""
-    want = DECODE_TARGET_WAVES // max(num_tokens * num_kv_heads, 1)
-    blocks = -(-max_seq_len // 16)
-    return max(1, min(want, DECODE_MAX_SPLITS, blocks))
+def decode_splits(num_tokens: int, num_kv_heads: int, max_seq_len: int, waves: int,
+                  window: int = 0) -> int:
+    """Into how many parts each request's key range is cut for the decode kernel, beyond
+    the ``waves`` waves of a block that share a part: one, unless a wave would walk more
+    than ``DECODE_BLOCKS_PER_WAVE`` blocks of 16 keys and the chip has room for more blocks."""
+    keys = max_seq_len if window <= 0 else min(max_seq_len, window + 16)
+    blocks = -(-keys // 16)
+    by_length = -(-blocks // (waves * DECODE_BLOCKS_PER_WAVE))
+    by_room = DECODE_TARGET_WAVES // max(num_tokens * num_kv_heads * waves, 1)
+    return max(1, min(by_length, by_room, DECODE_MAX_SPLITS))
 
 
 class PagedAttention(Mixer):
@@ -84,43 +89,47 @@ class PagedAttention(Mixer):
             rot_dim, interleaved = 0, False
         else:
             cos, sin, rot_dim, interleaved = rot.cos, rot.sin, rot.rot_dim, rot.interleaved
-        # where each token's key and value go: once per step and cache group
-        slot_key = ("kv_slot", call.group_index)
-        kv_slot = ctx.scratch.get(slot_key)
-        if kv_slot is None:
-            kv_slot = ctx.buf(f"kv_slot_{call.group_index}", 1, torch.int32).view(-1)
-            ops.kv_slots(kv_slot, positions=ctx.positions, token_req=ctx.token_req, slots=ctx.slots,
-                         table=group.table, page_size=group.page_size, num_pages=k_cache.shape[0])
-            ctx.scratch[slot_key] = kv_slot
-        ops.rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim, interleaved=interleaved,
-                          kv_slot=kv_slot, nh=self.num_heads, nkv=self.num_kv_heads,
-                          d=self.head_dim, write_kv=call.write_cache)
-
         attn = ctx.buf("attn_out", self.q_size)
         common = dict(table=group.table, positions=ctx.positions, token_req=ctx.token_req,
                       slots=ctx.slots, nh=self.num_heads, nkv=self.num_kv_heads, d=self.head_dim,
                       scale=self.scale, window=self.window)
         if ctx.max_query_len == 1 and ops.decode_attention_supported(
                 self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
-            # single tokens: one wave per (token, kv head, split) on the matrix cores
+            # single tokens: rotation, cache write and attention in one kernel on the matrix
+            # cores, a block per (token, kv head, split)
             T = ctx.num_tokens
-            nsplit = decode_splits(T, self.num_kv_heads, ctx.max_seq_len)
+            waves = ops.decode_attention_waves(self.num_heads, self.num_kv_heads, self.head_dim)
+            nsplit = decode_splits(T, self.num_kv_heads, ctx.max_seq_len, waves, self.window)
             part_o = part_ml = None
             if nsplit > 1:
                 part_o = ctx.buffers.get("attn_part_o", T * self.num_heads * nsplit, self.head_dim,
                                          torch.float32)
                 part_ml = ctx.buffers.get("attn_part_ml", T * self.num_heads * nsplit, 2, torch.float32)
             ops.decode_attention(attn, qkv, k_cache, v_cache, nsplit=nsplit, part_o=part_o,
-                                 part_ml=part_ml, **common)
-        elif ctx.max_query_len > 1 and ops.prefill_attention_supported(
-                self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
-            # portions of prompts (single tokens may ride along): tiles of query rows per block
-            ops.prefill_attention(attn, qkv, k_cache, v_cache, table=group.table,
-                                  positions=ctx.positions, q_start=ctx.q_start, slots=ctx.slots,
-                                  num_reqs=ctx.num_reqs, nh=self.num_heads, nkv=self.num_kv_heads,
-                                  d=self.head_dim, scale=self.scale, window=self.window)
+                                 part_ml=part_ml, cos=cos, sin=sin, rot_dim=rot_dim,
+                                 interleaved=interleaved, write_kv=call.write_cache, **common)
         else:
-            ops.paged_attention(attn, qkv, k_cache, v_cache, **common)
+            # where each token's key and value go: once per step and cache group
+            slot_key = ("kv_slot", call.group_index)
+            kv_slot = ctx.scratch.get(slot_key)
+            if kv_slot is None:
+                kv_slot = ctx.buf(f"kv_slot_{call.group_index}", 1, torch.int32).view(-1)
+                ops.kv_slots(kv_slot, positions=ctx.positions, token_req=ctx.token_req,
+                             slots=ctx.slots, table=group.table, page_size=group.page_size,
+                             num_pages=k_cache.shape[0])
+                ctx.scratch[slot_key] = kv_slot
+            ops.rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim,
+                              interleaved=interleaved, kv_slot=kv_slot, nh=self.num_heads,
+                              nkv=self.num_kv_heads, d=self.head_dim, write_kv=call.write_cache)
+            if ctx.max_query_len > 1 and ops.prefill_attention_supported(
+                    self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
+                # portions of prompts (single tokens may ride along): tiles of query rows per block
+                ops.prefill_attention(attn, qkv, k_cache, v_cache, table=group.table,
+                                      positions=ctx.positions, q_start=ctx.q_start, slots=ctx.slots,
+                                      num_reqs=ctx.num_reqs, nh=self.num_heads, nkv=self.num_kv_heads,
+                                      d=self.head_dim, scale=self.scale, window=self.window)
+            else:
+                ops.paged_attention(attn, qkv, k_cache, v_cache, **common)
         out = ctx.buf("mixer_out", self.hidden_size)
         ops.linear(out, attn, p["o_proj.weight"], p.get("o_proj.bias"))
         return out

@@ -36,10 +36,10 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx, call) -> torch.Tensor:
         p = self.params
-        gate_up = ctx.buf("ffn_gate_up", 2 * self.intermediate_size)
-        ops.linear(gate_up, x, p["gate_up_proj.weight"], p.get("gate_up_proj.bias"))
         act = ctx.buf("ffn_act", self.intermediate_size)
-        ops.silu_mul(act, gate_up)
+        # few rows: the product and the activation are one kernel and gate_up is never stored
+        ops.linear_silu_mul(act, x, p["gate_up_proj.weight"], p.get("gate_up_proj.bias"),
+                            lambda: ctx.buf("ffn_gate_up", 2 * self.intermediate_size))
         out = ctx.buf("ffn_out", self.hidden_size)
         ops.linear(out, act, p["down_proj.weight"], p.get("down_proj.bias"))
         return out

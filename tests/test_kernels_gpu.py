@@ -151,6 +151,35 @@ def test_gemm_skinny_bf16(ops, M, N, K, out_dtype):
     assert torch.equal(wide_out[:, :N], ref) and torch.all(wide_out[:, N:] == 0)
 
 
+@pytest.mark.parametrize("M,I,K", [(1, 16, 64), (5, 100, 200), (8, 2072, 512), (16, 88, 1032),
+                                   (17, 176, 80), (64, 40, 256)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_linear_silu_mul(ops, M, I, K, with_bias):
+    """The one-kernel form matches the formula, and gives the bits of the two-kernel form
+    (product stored in bfloat16, then the activation) where both split K the same way."""
+    x = rnd(M, K, dtype=torch.bfloat16, seed=1)
+    w = rnd(2 * I, K, dtype=torch.bfloat16, seed=2, scale=0.1)
+    bias = rnd(2 * I, dtype=torch.bfloat16, seed=3) if with_bias else None
+    out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    used_scratch = []
+
+    def scratch():
+        used_scratch.append(True)
+        return torch.empty(M, 2 * I, dtype=torch.bfloat16, device=DEV)
+
+    ops.linear_silu_mul(out, x, w, bias, scratch)
+    assert bool(used_scratch) == (M > 16)
+    gate_up = torch.empty(M, 2 * I, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_skinny_bf16(gate_up, x, w, bias)
+    two = torch.empty_like(out)
+    ops.silu_mul(two, gate_up)
+    if M <= 16 and 2 * I > 4096:
+        assert torch.equal(out, two)
+    gu = x.double() @ w.double().T + (bias.double() if with_bias else 0.0)
+    want = plain.silu_and_mul(gu)
+    assert torch.allclose(out.double(), want, atol=2e-2, rtol=2e-2)
+
+
 def test_linear_picks_a_kernel_by_row_count(ops):
     w = rnd(96, 256, dtype=torch.bfloat16, seed=5, scale=0.05)
     for M in (3, 64, 65, 200):
@@ -426,6 +455,66 @@ def test_decode_attention_on_the_matrix_cores(ops, nh, nkv, d, page, nsplit):
     ops.paged_attention(ref, q, kc, vc, table=table, positions=positions, token_req=token_req,
                         slots=slots, nh=nh, nkv=nkv, d=d, scale=scale)
     assert torch.allclose(out.float(), ref.float(), atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 1, 32, 16), (32, 8, 128, 16), (6, 2, 64, 32), (8, 2, 256, 16),
+                                           (3, 3, 96, 48), (16, 1, 160, 16)])
+@pytest.mark.parametrize("rot,interleaved", [("full", False), ("half", False), ("full", True), ("none", False)])
+@pytest.mark.parametrize("nsplit", [1, 3])
+def test_decode_attention_rotates_and_writes_like_the_separate_kernels(ops, nh, nkv, d, page, rot,
+                                                                        interleaved, nsplit):
+    """The decode kernel with rotation and cache write built in gives the bits of
+    rope_kv_write followed by the attention alone: outputs, and every byte of the cache."""
+    dtype = torch.bfloat16
+    seq_lens = [1, 15, 16, 17, 96, 97, 300, 641]
+    R = len(seq_lens)
+    kc, vc, table, dense = paged_setup(seq_lens, nkv, d, page, dtype, seed=d + nsplit)
+    for r, n in enumerate(seq_lens):  # the token's own slot is not written yet
+        pg, off = int(table[r + 1, (n - 1) // page]), (n - 1) % page
+        kc[pg, :, off] = float("nan")
+        vc[pg, :, :, off] = float("nan")
+    T = R + 1  # one padding token at the end
+    qkv0 = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=9)
+    positions = torch.tensor([n - 1 for n in seq_lens] + [0], dtype=torch.int32, device=DEV)
+    token_req = torch.tensor(list(range(R)) + [-1], dtype=torch.int32, device=DEV)
+    slots = torch.arange(1, R + 1, dtype=torch.int32, device=DEV)
+    rot_dim = {"full": d, "half": d // 2, "none": 0}[rot]
+    cos = torch.empty(T, rot_dim // 2, device=DEV)
+    sin = torch.empty(T, rot_dim // 2, device=DEV)
+    if rot_dim:
+        inv = plain.rope_inv_freq(rot_dim, 10000.0).float().to(DEV)
+        ops.rope_table(cos, sin, positions, inv)
+    part_o = torch.full((T * nh * nsplit, d), float("nan"), device=DEV)
+    part_ml = torch.full((T * nh * nsplit, 2), float("nan"), device=DEV)
+    common = dict(table=table, positions=positions, token_req=token_req, slots=slots, nh=nh, nkv=nkv,
+                  d=d, scale=d ** -0.5, nsplit=nsplit, part_o=part_o, part_ml=part_ml)
+
+    kc1, vc1, qkv1 = kc.clone(), vc.clone(), qkv0.clone()
+    kv_slot = torch.empty(T, dtype=torch.int32, device=DEV)
+    ops.kv_slots(kv_slot, positions=positions, token_req=token_req, slots=slots, table=table,
+                 page_size=page, num_pages=kc.shape[0])
+    ops.rope_kv_write(qkv1, kc1, vc1, cos, sin, rot_dim=rot_dim, interleaved=interleaved,
+                      kv_slot=kv_slot, nh=nh, nkv=nkv, d=d)
+    out1 = torch.full((T, nh * d), float("nan"), dtype=dtype, device=DEV)
+    ops.decode_attention(out1, qkv1, kc1, vc1, **common)
+    assert not torch.isnan(out1).any()
+
+    kc2, vc2, qkv2 = kc.clone(), vc.clone(), qkv0.clone()
+    out2 = torch.full((T, nh * d), float("nan"), dtype=dtype, device=DEV)
+    ops.decode_attention(out2, qkv2, kc2, vc2, cos=cos, sin=sin, rot_dim=rot_dim,
+                         interleaved=interleaved, write_kv=True, **common)
+    bits = lambda x: x.view(torch.int16)
+    assert torch.equal(bits(qkv2), bits(qkv0))
+    assert torch.equal(bits(out2), bits(out1))
+    assert torch.equal(bits(kc2), bits(kc1)) and torch.equal(bits(vc2), bits(vc1))
+
+    # without the write the cache must already hold the token (a layer that reads another's cache)
+    out3 = torch.full((T, nh * d), float("nan"), dtype=dtype, device=DEV)
+    kc3, vc3 = kc1.clone(), vc1.clone()
+    ops.decode_attention(out3, qkv0, kc3, vc3, cos=cos, sin=sin, rot_dim=rot_dim,
+                         interleaved=interleaved, write_kv=False, **common)
+    assert torch.equal(bits(out3), bits(out1))
+    assert torch.equal(bits(kc3), bits(kc1)) and torch.equal(bits(vc3), bits(vc1))
 
 
 @pytest.mark.parametrize("nsplit", [1, 5])
