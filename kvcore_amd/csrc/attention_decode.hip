@@ -59,6 +59,7 @@ struct DecodeArgs {
   const int32_t* positions;
   const int32_t* token_req;
   const int32_t* slots;
+  const int32_t* token_rows;  // [T] block-table row of each token (-1: padding), or null
   const float* cos_tab;  // [T, rot_dim / 2]
   const float* sin_tab;
   int rot_dim;
@@ -68,6 +69,7 @@ struct DecodeArgs {
   float scale_log2e;
   int window;
   int nsplit;
+  int lds_pages;  // page ids of a block's range that fit in LDS
 };
 
 __host__ __device__ inline size_t lds_q_bytes(int g, int d) {
@@ -78,8 +80,10 @@ __host__ __device__ inline size_t lds_ml_bytes(int waves) { return static_cast<s
 __host__ __device__ inline size_t lds_o_bytes(int waves, int g, int d) {
   return static_cast<size_t>(waves) * g * (d + kOPad) * 4;
 }
-inline size_t lds_total(int waves, int g, int d) {
-  return lds_q_bytes(g, d) + lds_kv_bytes(d) + lds_ml_bytes(waves) + lds_o_bytes(waves, g, d);
+constexpr int kMaxLdsPages = 1024;  // what the choice of waves per block leaves room for
+inline size_t lds_total(int waves, int g, int d, int lds_pages) {
+  return lds_q_bytes(g, d) + lds_kv_bytes(d) + lds_ml_bytes(waves) + lds_o_bytes(waves, g, d) +
+         static_cast<size_t>(lds_pages) * 4;
 }
 
 // wide heads keep more registers per lane, so fewer waves fit in a block
@@ -101,19 +105,29 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
   const int quad = lane >> 4;  // 0..3
   const int nh = a.nh, nkv = a.nkv, nsplit = a.nsplit, page_size = a.page_size;
   const int g = nh / nkv;
-  const int head = hk * g + col;
   const bool head_live = col < g;
   constexpr int NJ = D / 16;  // output row blocks
   constexpr int NC = D / 32;  // 32-wide chunks of the head for Q.K
+  constexpr int NBUF = 3;     // 16-key blocks a wave holds: one in work, two on their way
 
   bf16_t* sq = reinterpret_cast<bf16_t*>(lds);                       // [g][D + kQPad]
   bf16_t* sk = reinterpret_cast<bf16_t*>(lds + lds_q_bytes(g, D));   // [D] key, then [D] value
   bf16_t* sv = sk + D;
   float* sml = reinterpret_cast<float*>(lds + lds_q_bytes(g, D) + lds_kv_bytes(D));  // [waves][16][2]
   float* so = sml + waves * 32;                                      // [waves][g][D + kOPad]
+  int32_t* spage = reinterpret_cast<int32_t*>(so + static_cast<int64_t>(waves) * g * (D + kOPad));  // [lds_pages]
 
-  const int req = a.token_req[t];
-  if (req < 0) {  // padding token
+  // which row of the block table: one load if the caller resolved it, else two in a chain
+  const int pos = __builtin_amdgcn_readfirstlane(a.positions[t]);
+  int trow_idx;
+  if (a.token_rows != nullptr) {
+    trow_idx = a.token_rows[t];
+  } else {
+    const int req = a.token_req[t];
+    trow_idx = req < 0 ? -1 : a.slots[req];
+  }
+  trow_idx = __builtin_amdgcn_readfirstlane(trow_idx);
+  if (trow_idx < 0) {  // padding token
     if (nsplit == 1) {
       for (int idx = tid; idx < g * D; idx += nthreads)
         a.out[(static_cast<int64_t>(t) * nh + hk * g) * D + idx] = from_float<bf16_t>(0.f);
@@ -124,10 +138,9 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
     }
     return;
   }
-  const int pos = a.positions[t];
   const int window = a.window;
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int32_t* row = a.table + static_cast<int64_t>(a.slots[req]) * a.table_stride;
+  const int32_t* row = a.table + static_cast<int64_t>(trow_idx) * a.table_stride;
 
   // the 16-key blocks this block owns: [b0, b1) of the range that holds keys first..pos
   const int blk_first = first / 16;
@@ -138,6 +151,58 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
   const int b1 = (b0 + per < blk_end) ? b0 + per : blk_end;
   const int blk_own = pos / 16;  // the block of the token's own key
   const bool owner = a.write_kv && b0 <= blk_own && blk_own < b1;
+  const int blocks_per_page = page_size / 16;
+
+  // the page ids of the range go to LDS, where the walk below reads them
+  const int page_lo = b0 / blocks_per_page;
+  const int n_range_pages = (b1 > b0) ? (b1 - 1) / blocks_per_page - page_lo + 1 : 0;
+  for (int i = tid; i < n_range_pages && i < a.lds_pages; i += nthreads)
+    spage[i] = (page_lo + i < a.table_stride) ? row[page_lo + i] : 0;
+
+  // One 16-key block: K rows as A operand (row = key `col`, elements 32c + 8*quad .. +8) and
+  // V^T rows (row = element 16j + col, keys 4*quad .. +4).  The loads are issued without any
+  // branch around them, so that the waits the compiler places count them exactly and a
+  // block's loads stay in flight while earlier blocks are worked on.
+  bf16x8_t kb[NBUF][NC];
+  s16x4_t vb[NBUF][NJ];
+  bool okb[NBUF];
+  auto issue_block = [&](int bn, int page, bf16x8_t (&ka)[NC], s16x4_t (&va)[NJ]) -> bool {
+    const bool in_range = bn < b1;
+    const bool page_ok = page > 0 && page < a.num_pages;  // else given back behind the window
+    const bool real = in_range && page_ok;
+    const int sub = bn % blocks_per_page;
+    // a block that is not there reads one line of the null page with every lane
+    const bf16_t* krow = real ? a.k_cache + ((static_cast<int64_t>(page) * nkv + hk) * page_size +
+                                             sub * 16 + col) * D + 8 * quad
+                              : a.k_cache;
+    const bf16_t* vrow = real ? a.v_cache + ((static_cast<int64_t>(page) * nkv + hk) * D + col) * page_size +
+                                    sub * 16 + 4 * quad
+                              : a.v_cache;
+    const int64_t v_step = real ? static_cast<int64_t>(16) * page_size : 0;
+    const int k_step = real ? 32 : 0;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) ka[c] = *reinterpret_cast<const bf16x8_t*>(krow + k_step * c);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) va[j] = *reinterpret_cast<const s16x4_t*>(vrow + v_step * j);
+    return real;
+  };
+  auto clamp_block = [&](int bn) -> int { return bn < b1 ? bn : b1 - 1; };
+
+  // the first blocks of this wave are asked for at once, before anything else waits
+  const int b_wave = b0 + wave;
+  const bool has_work = b_wave < b1;
+#pragma unroll
+  for (int s = 0; s < NBUF; ++s) okb[s] = false;
+  if (has_work) {
+    int first_pages[NBUF - 1];
+#pragma unroll
+    for (int s = 0; s < NBUF - 1; ++s) {
+      const int page_idx = clamp_block(b_wave + s * waves) / blocks_per_page;
+      first_pages[s] = __builtin_amdgcn_readfirstlane((page_idx < a.table_stride) ? row[page_idx] : 0);
+    }
+#pragma unroll
+    for (int s = 0; s < NBUF - 1; ++s) okb[s] = issue_block(b_wave + s * waves, first_pages[s], kb[s], vb[s]);
+  }
 
   // ---- rotation of the group's queries (and the key) into LDS; key and value into the cache
   {
@@ -212,115 +277,92 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
   for (int j = 0; j < NJ; ++j) o[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  const int blocks_per_page = page_size / 16;
-  // one 16-key block: K rows as A operand (row = key `col`, elements 32c + 8*quad .. +8) and
-  // V^T rows (row = element 16j + col, keys 4*quad .. +4)
-  auto load_block = [&](int b, bf16x8_t (&ka)[NC], s16x4_t (&va)[NJ]) -> bool {
-    const int page_idx = b / blocks_per_page;
-    const int sub = b - page_idx * blocks_per_page;
-    const int page = (page_idx < a.table_stride) ? row[page_idx] : 0;
-    if (page <= 0 || page >= a.num_pages) return false;  // a page given back behind the window
-    const bf16_t* krow = a.k_cache +
-                         ((static_cast<int64_t>(page) * nkv + hk) * page_size + sub * 16 + col) * D + 8 * quad;
-    const bf16_t* vrow = a.v_cache + ((static_cast<int64_t>(page) * nkv + hk) * D + col) * page_size +
-                         sub * 16 + 4 * quad;
+  auto work_block = [&](int b, bf16x8_t (&ka)[NC], s16x4_t (&va)[NJ]) {
+    if (owner && b == blk_own) {
+      // the token's own key and value come from LDS, not from the cache line just written
+      const int kk = pos & 15;
+      if (col == kk) {
 #pragma unroll
-    for (int c = 0; c < NC; ++c) ka[c] = *reinterpret_cast<const bf16x8_t*>(krow + 32 * c);
-#pragma unroll
-    for (int j = 0; j < NJ; ++j)
-      va[j] = *reinterpret_cast<const s16x4_t*>(vrow + static_cast<int64_t>(16 * j) * page_size);
-    return true;
-  };
-
-  bf16x8_t k_cur[NC], k_next[NC];
-  s16x4_t v_cur[NJ], v_next[NJ];
-#pragma unroll
-  for (int c = 0; c < NC; ++c) k_next[c] = bq[c];
-#pragma unroll
-  for (int j = 0; j < NJ; ++j) v_next[j] = s16x4_t{0, 0, 0, 0};
-  bool ok_cur = false, ok_next = false;
-  int b = b0 + wave;
-  if (b < b1) ok_cur = load_block(b, k_cur, v_cur);
-  for (; b < b1; b += waves) {
-    const int bn = b + waves;
-    if (bn < b1) ok_next = load_block(bn, k_next, v_next);
-    if (ok_cur) {
-      if (owner && b == blk_own) {
-        // the token's own key and value come from LDS, not from the cache line just written
-        const int kk = pos & 15;
-        if (col == kk) {
-#pragma unroll
-          for (int c = 0; c < NC; ++c)
-            k_cur[c] = *reinterpret_cast<const bf16x8_t*>(sk + 32 * c + 8 * quad);
-        }
-        if (quad == (kk >> 2)) {
-#pragma unroll
-          for (int j = 0; j < NJ; ++j) {
-            const short bits = static_cast<short>(sv[16 * j + col].bits);
-            if ((kk & 3) == 0) v_cur[j][0] = bits;
-            if ((kk & 3) == 1) v_cur[j][1] = bits;
-            if ((kk & 3) == 2) v_cur[j][2] = bits;
-            if ((kk & 3) == 3) v_cur[j][3] = bits;
-          }
-        }
+        for (int c = 0; c < NC; ++c) ka[c] = *reinterpret_cast<const bf16x8_t*>(sk + 32 * c + 8 * quad);
       }
-      f32x4_t s = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (quad == (kk >> 2)) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_cur[c], bq[c], s, 0, 0, 0);
-
-      // s[i] belongs to key 16b + 4*quad + i and head `col`
-      const int key0 = 16 * b + 4 * quad;
-      float sv4[4];
-      bool ok[4];
-      float mx = -INFINITY;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = key0 + i;
-        ok[i] = key >= first && key <= pos;
-        sv4[i] = ok[i] ? s[i] * a.scale_log2e : -INFINITY;
-        mx = fmaxf(mx, sv4[i]);
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m, mx);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
-      float p[4];
-      float ps = 0.f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        p[i] = __builtin_amdgcn_exp2f(sv4[i] - m_safe);  // exp2(-inf) = 0 for masked keys
-        ps += p[i];
-      }
-      ps += __shfl_xor(ps, 16, 64);
-      ps += __shfl_xor(ps, 32, 64);
-      l = l * alpha + ps;
-      m = m_new;
-
-      // P^T as B operand of the 16x16x16 product: k = key 4*quad + i, column = head
-      s16x4_t pb;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) pb[i] = static_cast<short>(f32_to_bf16_bits(p[i]));
-      // values of masked keys may be anything (a reused page, NaN): they must not meet the
-      // product even with weight zero
-      const bool edge = (16 * b + 15 > pos) || (16 * b < first);
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        s16x4_t va = v_cur[j];
-        if (edge) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (!ok[i]) va[i] = 0;
+        for (int j = 0; j < NJ; ++j) {
+          const short bits = static_cast<short>(sv[16 * j + col].bits);
+          if ((kk & 3) == 0) va[j][0] = bits;
+          if ((kk & 3) == 1) va[j][1] = bits;
+          if ((kk & 3) == 2) va[j][2] = bits;
+          if ((kk & 3) == 3) va[j][3] = bits;
         }
-        o[j] = o[j] * alpha;
-        o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb, o[j], 0, 0, 0);
       }
     }
+    f32x4_t s = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < NC; ++c) k_cur[c] = k_next[c];
+    for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], bq[c], s, 0, 0, 0);
+
+    // s[i] belongs to key 16b + 4*quad + i and head `col`
+    const int key0 = 16 * b + 4 * quad;
+    float sv4[4];
+    bool ok[4];
+    float mx = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) v_cur[j] = v_next[j];
-    ok_cur = ok_next;
+    for (int i = 0; i < 4; ++i) {
+      const int key = key0 + i;
+      ok[i] = key >= first && key <= pos;
+      sv4[i] = ok[i] ? s[i] * a.scale_log2e : -INFINITY;
+      mx = fmaxf(mx, sv4[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+    float p[4];
+    float ps = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = __builtin_amdgcn_exp2f(sv4[i] - m_safe);  // exp2(-inf) = 0 for masked keys
+      ps += p[i];
+    }
+    ps += __shfl_xor(ps, 16, 64);
+    ps += __shfl_xor(ps, 32, 64);
+    l = l * alpha + ps;
+    m = m_new;
+
+    // P^T as B operand of the 16x16x16 product: k = key 4*quad + i, column = head
+    s16x4_t pb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pb[i] = static_cast<short>(f32_to_bf16_bits(p[i]));
+    // values of masked keys may be anything (a reused page, NaN): they must not meet the
+    // product even with weight zero
+    const bool edge = (16 * b + 15 > pos) || (16 * b < first);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      s16x4_t vv = va[j];
+      if (edge) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (!ok[i]) vv[i] = 0;
+      }
+      o[j] = o[j] * alpha;
+      o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vv, pb, o[j], 0, 0, 0);
+    }
+  };
+
+  // the wave's blocks b_wave, b_wave + waves, ...: while one is worked on, the next two load
+  if (has_work) {
+    for (int b = b_wave; b < b1; b += NBUF * waves) {
+#pragma unroll
+      for (int s = 0; s < NBUF; ++s) {
+        const int bc = b + s * waves;
+        constexpr int kAhead = NBUF - 1;
+        const int bn = bc + kAhead * waves;
+        const int sn = (s + kAhead) % NBUF;
+        const int page = __builtin_amdgcn_readfirstlane(spage[clamp_block(bn) / blocks_per_page - page_lo]);
+        okb[sn] = issue_block(bn, page, kb[sn], vb[sn]);
+        if (bc < b1 && okb[s]) work_block(bc, kb[s], vb[s]);  // the same for the whole wave
+      }
+    }
   }
 
   // ---- merge the waves' partials in wave order
@@ -362,56 +404,67 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
   }
 }
 
-// out[t, head, :] = sum_s w_s * part_o[s] / sum_s w_s * l_s with w_s = exp2(m_s - max m)
+// out[t, head, :] = sum_s w_s * part_o[s] / sum_s w_s * l_s with w_s = exp2(m_s - max m).
+// Every wave works the weights out for itself (lane s holds split s), so nothing waits on
+// another wave; the partial outputs are asked for before the weights are known.
+constexpr int kMaxSplits = 64;
 __global__ void decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                                       const float* __restrict__ part_ml, int D, int nsplit) {
-  extern __shared__ float wgt[];  // [nsplit]
-  __shared__ float inv_denom;
   const int64_t th = blockIdx.x;  // token * nh + head
+  const int lane = threadIdx.x & 63;
   const float* ml = part_ml + th * nsplit * 2;
-  if (threadIdx.x < 64) {  // the first wave: weights of the splits
-    float mmax = -INFINITY;
-    for (int s = threadIdx.x; s < nsplit; s += 64) mmax = fmaxf(mmax, ml[2 * s]);
-    mmax = wave_max(mmax);
-    const float m_safe = (mmax == -INFINITY) ? 0.f : mmax;
-    for (int s = threadIdx.x; s < nsplit; s += 64) wgt[s] = __builtin_amdgcn_exp2f(ml[2 * s] - m_safe);
+  const float* po = part_o + th * nsplit * D;
+  float m_s = -INFINITY, l_s = 0.f;
+  if (lane < nsplit) {
+    m_s = ml[2 * lane];
+    l_s = ml[2 * lane + 1];
   }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float denom = 0.f;
-    for (int s = 0; s < nsplit; ++s) denom += wgt[s] * ml[2 * s + 1];
-    inv_denom = (denom > 0.f) ? 1.f / denom : 0.f;
-  }
-  __syncthreads();
-  const float inv = inv_denom;
-  for (int e = threadIdx.x; e < D; e += blockDim.x) {
+  for (int e0 = 0; e0 < D; e0 += blockDim.x) {
+    const int e = e0 + threadIdx.x;
+    const bool live = e < D;
     float acc = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float w = wgt[s];
-      if (w > 0.f) acc += w * part_o[(th * nsplit + s) * D + e];
+    float mmax = wave_max(m_s);
+    const float m_safe = (mmax == -INFINITY) ? 0.f : mmax;
+    const float w_lane = __builtin_amdgcn_exp2f(m_s - m_safe);  // 0 for lanes beyond nsplit
+    const float denom = wave_sum(w_lane * l_s);
+    for (int s0 = 0; s0 < nsplit; s0 += 4) {
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        v[i] = (live && s0 + i < nsplit) ? po[static_cast<int64_t>(s0 + i) * D + e] : 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float w = __shfl(w_lane, (s0 + i) & 63, 64);
+        if (s0 + i < nsplit && w > 0.f) acc += w * v[i];
+      }
     }
-    out[th * D + e] = from_float<bf16_t>(acc * inv);
+    if (live) out[th * D + e] = from_float<bf16_t>(denom > 0.f ? acc / denom : 0.f);
   }
 }
 
 int decode_waves(int g, int d) {
   int waves = d > 128 ? 4 : kMaxWaves;
-  while (waves > 1 && lds_total(waves, g, d) > kLdsLimit) waves /= 2;
+  while (waves > 1 && lds_total(waves, g, d, kMaxLdsPages) > kLdsLimit) waves /= 2;
   return waves;
 }
 
 template <int D>
-int launch_decode(const DecodeArgs& args, int T, hipStream_t stream) {
+int launch_decode(DecodeArgs& args, int T, hipStream_t stream) {
   const int g = args.nh / args.nkv;
+  // a split's range of pages always fits: the table's width cut into nsplit parts, and slack
+  args.lds_pages = (args.table_stride + args.nsplit - 1) / args.nsplit + 2;
+  if (args.lds_pages > args.table_stride) args.lds_pages = args.table_stride;
   int waves = decode_waves(g, D);
   // more blocks than compute units: smaller blocks pack better
   if (static_cast<int64_t>(T) * args.nkv * args.nsplit > 256 && waves > 4) waves = 4;
+  while (waves > 1 && lds_total(waves, g, D, args.lds_pages) > kLdsLimit) waves /= 2;
+  if (lds_total(waves, g, D, args.lds_pages) > kLdsLimit)
+    return kvc_fail("kvc_decode_attention: the block table is too wide for one split (use more)");
   hipLaunchKernelGGL(decode_attention_kernel<D>, dim3(T, args.nkv, args.nsplit), dim3(waves * 64),
-                     lds_total(waves, g, D), stream, args);
+                     lds_total(waves, g, D, args.lds_pages), stream, args);
   if (args.nsplit > 1)
-    hipLaunchKernelGGL(decode_combine_kernel, dim3(T * args.nh), dim3(D < 64 ? 64 : D),
-                       args.nsplit * sizeof(float), stream, args.out, args.part_o, args.part_ml, D,
-                       args.nsplit);
+    hipLaunchKernelGGL(decode_combine_kernel, dim3(T * args.nh), dim3((D + 63) / 64 * 64), 0, stream,
+                       args.out, args.part_o, args.part_ml, D, args.nsplit);
   return kvc_check_launch("kvc_decode_attention");
 }
 
@@ -433,15 +486,15 @@ extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, cons
                                     int64_t qkv_stride, void* k_cache, void* v_cache,
                                     const int32_t* table, int table_stride,
                                     const int32_t* positions, const int32_t* token_req,
-                                    const int32_t* slots, const float* cos_tab, const float* sin_tab,
-                                    int rot_dim, int interleaved, int write_kv, int T, int nh,
+                                    const int32_t* slots, const int32_t* token_rows,
+                                    const float* cos_tab, const float* sin_tab, int rot_dim, int interleaved, int write_kv, int T, int nh,
                                     int nkv, int d, int page_size, int num_pages, float scale,
                                     int window, int nsplit, kvc_stream stream) {
   if (!kvc_decode_attention_supported(nh, nkv, d, page_size, 1))
     return kvc_fail("kvc_decode_attention: unsupported shape (bfloat16, head size a multiple of 32 "
                     "up to 256, at most 16 query heads per kv head, page size a multiple of 16)");
-  if (T < 0 || nsplit < 1 || nsplit > 65535 || nkv > 65535 || table_stride <= 0 || num_pages <= 0)
-    return kvc_fail("kvc_decode_attention: bad sizes");
+  if (T < 0 || nsplit < 1 || nsplit > kMaxSplits || nkv > 65535 || table_stride <= 0 || num_pages <= 0)
+    return kvc_fail("kvc_decode_attention: bad sizes (at most 64 splits)");
   if (qkv_stride % 8 || qkv_stride < static_cast<int64_t>(nh + (write_kv ? 2 * nkv : 0)) * d)
     return kvc_fail("kvc_decode_attention: token rows must be 16-byte aligned and hold q (and k, v)");
   if (rot_dim < 0 || rot_dim > d || rot_dim % 2)
@@ -464,6 +517,7 @@ extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, cons
   args.positions = positions;
   args.token_req = token_req;
   args.slots = slots;
+  args.token_rows = token_rows;
   args.cos_tab = cos_tab;
   args.sin_tab = sin_tab;
   args.rot_dim = rot_dim;

@@ -65,7 +65,10 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
                                    int M, int N, int K, int64_t lda, int64_t ldc, int k_per_wave) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
   extern __shared__ float red[];  // [waves - 1][RT * NT][64][4]
-  const int wave = threadIdx.x >> 6;
+  // wave-uniform values are made scalar on purpose: a condition on them becomes a scalar
+  // branch, and matrix instructions are only ever skipped by branches (they do not honour
+  // the lane mask that a vector condition would leave)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int waves = blockDim.x >> 6;
   const int lane = threadIdx.x & 63;
   const int col = lane & 15;
@@ -95,13 +98,15 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // Whole steps of 64 along K first, software-pipelined: the loads of step i+1 are issued
-  // before the products of step i, so every wave always has a step's worth of 16-byte
-  // loads in flight (a lane reads 2 x 16 bytes = a row reads 128 contiguous bytes a
-  // step).  Then whole 32-wide steps, then one guarded step for a tail (a multiple of 8).
+  // Whole steps of 64 along K first, software-pipelined: the loads of the next STAGES - 1
+  // steps are in flight while a step is multiplied (a lane reads 2 x 16 bytes = a row reads
+  // 128 contiguous bytes a step).  Then whole 32-wide steps, then one guarded step for a
+  // tail (a multiple of 8).
   constexpr int STAGES = U;  // steps in flight, the one being multiplied included
   bf16x8_t abuf[STAGES][RT][2], bbuf[STAGES][NT][2];
-  auto load_step = [&](int stage, int k) {
+  const int n64 = (k_end - k_begin) / 64;
+  auto load_step = [&](int stage, int step) {
+    const int k = k_begin + 64 * step;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       abuf[stage][rt][0] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k);
@@ -123,16 +128,18 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
           acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(abuf[stage][rt][h], bbuf[stage][nt][h],
                                                                  acc[rt][nt], 0, 0, 0);
   };
-  const int n64 = (k_end - k_begin) / 64;
+  // (Loads without a branch around them would let the waits count them exactly and keep
+  // all STAGES steps in flight; measured inside a decode step that is slower than this form,
+  // whose waits drain more often but which needs fewer registers and so runs more waves.)
   int k = k_begin;
 #pragma unroll
   for (int st = 0; st < STAGES - 1; ++st)
-    if (st < n64) load_step(st, k_begin + 64 * st);
+    if (st < n64) load_step(st, st);
   for (int i = 0; i < n64; i += STAGES) {
 #pragma unroll
     for (int j = 0; j < STAGES; ++j) {
-      if (i + j < n64) {  // uniform
-        if (i + j + STAGES - 1 < n64) load_step((j + STAGES - 1) % STAGES, k_begin + 64 * (i + j + STAGES - 1));
+      if (i + j < n64) {  // the same for the whole wave, and a scalar branch
+        if (i + j + STAGES - 1 < n64) load_step((j + STAGES - 1) % STAGES, i + j + STAGES - 1);
         mma_step(j);
       }
     }
@@ -244,8 +251,8 @@ void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M
 }
 
 // The launch shape is a function of N and K alone, so that a row's sums do not depend on
-// how many rows come with it.  Measured on MI355X at 1 to 16 rows: outputs wider than 4096
-// want 32 weight rows a wave and 4 waves along K, narrower ones 16 rows and 8 waves.
+// how many rows come with it.  Measured on MI355X at 1 to 16 rows: 4 waves along K; outputs
+// wider than 4096 want 32 weight rows a wave, narrower ones 16.
 // KVC_SKINNY_RT / KVC_SKINNY_WAVES override the choice for tuning.
 inline void pick_shape(int N, int K, int* rt_out, int* waves_out) {
   int rt, waves;
@@ -254,7 +261,7 @@ inline void pick_shape(int N, int K, int* rt_out, int* waves_out) {
     waves = 4;
   } else {
     rt = 1;
-    waves = 8;
+    waves = 4;
   }
   while (waves > 1 && K / waves < 128) waves /= 2;
   if (const char* e = getenv("KVC_SKINNY_RT")) rt = atoi(e);

@@ -85,6 +85,8 @@ int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* 
 // [T, nh, nsplit, 2] float32; a second kernel combines the splits (a "last block combines"
 // scheme needs device-scope fences, which on this chip write back and invalidate a whole L2
 // slice per block and cost more than the launch they save).
+// token_rows [T], if not null, holds slots[token_req[t]] (-1 for padding) and saves the
+// kernel one dependent load.
 // kvc_decode_attention_supported tells whether a shape is served (else use
 // kvc_paged_attention); kvc_decode_attention_waves how many waves share a block's key range.
 int kvc_decode_attention_supported(int nh, int nkv, int d, int page_size, int dtype);
@@ -92,10 +94,10 @@ int kvc_decode_attention_waves(int nh, int nkv, int d);
 int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* qkv,
                          int64_t qkv_stride, void* k_cache, void* v_cache, const int32_t* table,
                          int table_stride, const int32_t* positions, const int32_t* token_req,
-                         const int32_t* slots, const float* cos_tab, const float* sin_tab,
-                         int rot_dim, int interleaved, int write_kv, int T, int nh, int nkv, int d,
-                         int page_size, int num_pages, float scale, int window, int nsplit,
-                         kvc_stream stream);
+                         const int32_t* slots, const int32_t* token_rows, const float* cos_tab,
+                         const float* sin_tab, int rot_dim, int interleaved, int write_kv, int T,
+                         int nh, int nkv, int d, int page_size, int num_pages, float scale,
+                         int window, int nsplit, kvc_stream stream);
 
 // The same attention for bfloat16 portions of prompts on the matrix cores: a block per
 // (tile of a request's tokens, kv head), keys staged through LDS.  q_start [R+1] bounds

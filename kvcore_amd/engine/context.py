@@ -89,7 +89,8 @@ class StepContext:
 
     ``token_req[t]`` is the index of token ``t``'s request within this step (−1 marks a
     padding token); ``slots[r]`` is request ``r``'s slot: its row in every block table
-    and state array.  ``seq_lens[r]`` counts the request's tokens after this step,
+    and state array (``token_rows[t]``, if given, is ``slots[token_req[t]]``, −1 for
+    padding).  ``seq_lens[r]`` counts the request's tokens after this step,
     ``q_start[r] .. q_start[r+1]`` are its tokens in the flattened batch.
     """
 
@@ -112,6 +113,7 @@ class StepContext:
     max_query_len: int = 0
     max_seq_len: int = 0
     scratch: dict = field(default_factory=dict)  # per-step values parts share (rotary tables)
+    token_rows: torch.Tensor | None = None
 
     def buf(self, name: str, cols: int, dtype: torch.dtype | None = None, rows: int | None = None) -> torch.Tensor:
         return self.buffers.get(name, self.num_tokens if rows is None else rows, cols,

@@ -138,8 +138,8 @@ class ModelRunner:
         # packed per-step metadata: fixed layout, one upload
         T, R = max_num_tokens, max_num_seqs
         self._upd_cap = 2 * (T + R)
-        sections = [("token_ids", T), ("positions", T), ("token_req", T), ("logit_rows", T),
-                    ("q_start", R + 1), ("seq_lens", R), ("slots", R)]
+        sections = [("token_ids", T), ("positions", T), ("token_req", T), ("token_rows", T),
+                    ("logit_rows", T), ("q_start", R + 1), ("seq_lens", R), ("slots", R)]
         self._off: dict[str, tuple[int, int]] = {}
         cursor = 0
         for name, n in sections:
@@ -260,6 +260,7 @@ class ModelRunner:
             npv["token_ids"][:R] = toks
             npv["positions"][:R] = starts
             npv["token_req"][:R] = self._arange[:R]
+            npv["token_rows"][:R] = slot_list
             npv["q_start"][:R + 1] = self._arange[:R + 1]
             npv["seq_lens"][:R] = starts
             npv["seq_lens"][:R] += 1
@@ -297,6 +298,7 @@ class ModelRunner:
             npv["token_ids"][t:t + n] = toks
             npv["positions"][t:t + n] = np.arange(e.start, end, dtype=np.int32)
             npv["token_req"][t:t + n] = r
+            npv["token_rows"][t:t + n] = e.slot
             npv["q_start"][r] = t
             npv["seq_lens"][r] = end
             npv["slots"][r] = e.slot
@@ -321,6 +323,7 @@ class ModelRunner:
             npv["token_ids"][R:bucket] = 0
             npv["positions"][R:bucket] = 0
             npv["token_req"][R:bucket] = -1
+            npv["token_rows"][R:bucket] = -1
             npv["logit_rows"][:bucket] = np.arange(bucket, dtype=np.int32)
             npv["q_start"][R:bucket + 1] = np.arange(R, bucket + 1, dtype=np.int32)
             npv["seq_lens"][R:bucket] = 0
@@ -359,7 +362,8 @@ class ModelRunner:
         return StepContext(
             num_tokens=T, num_reqs=R,
             token_ids=self._dev["token_ids"], positions=self._dev["positions"],
-            token_req=self._dev["token_req"], q_start=self._dev["q_start"],
+            token_req=self._dev["token_req"], token_rows=self._dev["token_rows"],
+            q_start=self._dev["q_start"],
             seq_lens=self._dev["seq_lens"], slots=self._dev["slots"],
             groups=self.groups, states=self.states, buffers=self.buffers,
             dtype=self.dtype, device=self.device,

@@ -40,7 +40,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
         "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, P],
         "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
-        "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
+        "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
                                  F, I, I, P],
         "kvc_decode_attention_waves": [I, I, I],
         "kvc_decode_attention_supported": [I, I, I, I, I],
@@ -267,11 +267,12 @@ def decode_attention(out: torch.Tensor, qkv: torch.Tensor, k_cache: torch.Tensor
                      nsplit: int = 1, part_o: torch.Tensor | None = None,
                      part_ml: torch.Tensor | None = None, cos: torch.Tensor | None = None,
                      sin: torch.Tensor | None = None, rot_dim: int = 0, interleaved: bool = False,
-                     write_kv: bool = False) -> None:
+                     write_kv: bool = False, token_rows: torch.Tensor | None = None) -> None:
     """bfloat16 attention of single tokens on the matrix cores (see the C header), with the
     rotation of each token's query and key and the write of its key and value into the cache
     (``write_kv``) in the same kernel; ``qkv`` is not changed.  With ``rot_dim = 0`` and
-    ``write_kv = False`` it is the attention alone over queries as they are.  ``part_o`` and
+    ``write_kv = False`` it is the attention alone over queries as they are.  ``token_rows``
+    (``slots[token_req]``, -1 for padding) may be given to save the kernel a lookup.  ``part_o`` and
     ``part_ml`` are float32 workspaces of at least ``T*nh*nsplit*d`` and ``T*nh*nsplit*2``
     elements when ``nsplit > 1``."""
     T = out.shape[0]
@@ -301,7 +302,9 @@ def decode_attention(out: torch.Tensor, qkv: torch.Tensor, k_cache: torch.Tensor
         out.data_ptr(), po, pm, qkv.data_ptr(), qkv.stride(0), _dev(k_cache, "k_cache"),
         _dev(v_cache, "v_cache"), _dev(table, "table", torch.int32), table.shape[1],
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
-        _dev(slots, "slots", torch.int32), c, s_, int(rot_dim), int(bool(interleaved)),
+        _dev(slots, "slots", torch.int32),
+        None if token_rows is None else _dev(token_rows, "token_rows", torch.int32),
+        c, s_, int(rot_dim), int(bool(interleaved)),
         int(bool(write_kv)), T, nh, nkv, d, page_size, num_pages, float(scale),
         int(window), int(nsplit), _stream()), "kvc_decode_attention")
 

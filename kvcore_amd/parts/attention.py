@@ -15,21 +15,21 @@ from kvcore_amd.ops import library as ops
 from .base import CacheNeed, Mixer, ParamSource, ParamSpec, PositionEncoding, register_mixer
 
 
-DECODE_TARGET_WAVES = 1024  # enough waves to keep 256 compute units fed
+DECODE_TARGET_BLOCKS = 256  # one block for each compute unit
 DECODE_MAX_SPLITS = 32
-DECODE_BLOCKS_PER_WAVE = 8  # 16-key blocks one wave may walk before the range is split
 
 
 def decode_splits(num_tokens: int, num_kv_heads: int, max_seq_len: int, waves: int,
                   window: int = 0) -> int:
-    """Into how many parts each request's key range is cut for the decode kernel, beyond
-    the ``waves`` waves of a block that share a part: one, unless a wave would walk more
-    than ``DECODE_BLOCKS_PER_WAVE`` blocks of 16 keys and the chip has room for more blocks."""
+    """Into how many parts each request's key range is cut for the decode kernel, beyond the
+    ``waves`` waves of a block that share a part.  One compute unit draws keys and values
+    from memory far slower than the chip can deliver them, so the parts are made many
+    enough to occupy every unit, as long as each wave still has a block of 16 keys."""
     keys = max_seq_len if window <= 0 else min(max_seq_len, window + 16)
     blocks = -(-keys // 16)
-    by_length = -(-blocks // (waves * DECODE_BLOCKS_PER_WAVE))
-    by_room = DECODE_TARGET_WAVES // max(num_tokens * num_kv_heads * waves, 1)
-    return max(1, min(by_length, by_room, DECODE_MAX_SPLITS))
+    by_room = -(-DECODE_TARGET_BLOCKS // max(num_tokens * num_kv_heads, 1))
+    by_length = max(1, blocks // waves)
+    return max(1, min(by_room, by_length, DECODE_MAX_SPLITS))
 
 
 class PagedAttention(Mixer):
@@ -107,7 +107,8 @@ class PagedAttention(Mixer):
                 part_ml = ctx.buffers.get("attn_part_ml", T * self.num_heads * nsplit, 2, torch.float32)
             ops.decode_attention(attn, qkv, k_cache, v_cache, nsplit=nsplit, part_o=part_o,
                                  part_ml=part_ml, cos=cos, sin=sin, rot_dim=rot_dim,
-                                 interleaved=interleaved, write_kv=call.write_cache, **common)
+                                 interleaved=interleaved, write_kv=call.write_cache,
+                                 token_rows=ctx.token_rows, **common)
         else:
             # where each token's key and value go: once per step and cache group
             slot_key = ("kv_slot", call.group_index)

@@ -501,8 +501,10 @@ def test_decode_attention_rotates_and_writes_like_the_separate_kernels(ops, nh, 
 
     kc2, vc2, qkv2 = kc.clone(), vc.clone(), qkv0.clone()
     out2 = torch.full((T, nh * d), float("nan"), dtype=dtype, device=DEV)
+    token_rows = torch.tensor(list(range(1, R + 1)) + [-1], dtype=torch.int32, device=DEV)
     ops.decode_attention(out2, qkv2, kc2, vc2, cos=cos, sin=sin, rot_dim=rot_dim,
-                         interleaved=interleaved, write_kv=True, **common)
+                         interleaved=interleaved, write_kv=True,
+                         token_rows=token_rows if nsplit == 1 else None, **common)
     bits = lambda x: x.view(torch.int16)
     assert torch.equal(bits(qkv2), bits(qkv0))
     assert torch.equal(bits(out2), bits(out1))
