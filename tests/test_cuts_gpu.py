@@ -219,3 +219,29 @@ def collect_one(session, rec, starts):
         starts[item["id"]] = offsets[item["id"]] + len(item["tokens"])
     session.manager.check()
     return got
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
+def test_decoding_across_a_length_class(models, dtype):
+    """A long request decodes from 1000 to 1100 tokens beside a short one.  Steps of single
+    tokens are captured as graphs per class of sequence length (up to 1024, up to 2048, ...)
+    and the decode kernel cuts the key range by that class, so the step that crosses 1024
+    changes both; the short request's key range is then shorter than the number of parts."""
+    folder, cfg, weights, page = models["D"]
+    long_tokens = random_tokens(1100, cfg["vocab_size"], seed=501)
+    short_tokens = random_tokens(130, cfg["vocab_size"], seed=502)
+    session = session_for(folder, dtype, page, max_tokens=1100 + 192)
+    steps = [{"step": 0, "entries": [{"id": "L", "tokens": long_tokens[:1000], "want": [999]},
+                                     {"id": "S", "tokens": short_tokens[:30], "want": [29]}], "end": []}]
+    for j in range(100):
+        steps.append({"step": j + 1, "entries": [
+            {"id": "L", "tokens": [long_tokens[1000 + j]], "want": [0]},
+            {"id": "S", "tokens": [short_tokens[30 + j]], "want": [0]}], "end": []})
+    got = collect(session, steps)
+    assert len(got) == 202
+    compare(got, {"L": oracle("D", cfg, weights, long_tokens),
+                  "S": oracle("D", cfg, weights, short_tokens)}, dtype)
+    if session.runner.use_hip_graphs:
+        assert session.runner.graph_replays >= 90  # two classes, each: one step eager, one captured
+        # the longer class is there (the shorter one's graph goes when a step buffer grows)
+        assert -(-(1100 + 192) // 64) * 64 in {key[1] for key in session.runner._graphs}
