@@ -3,15 +3,18 @@
 // A block of four waves owns up to 64*CT query rows of one request and one kv head:
 // BQ = 64*CT / g consecutive tokens times the g query heads that share the kv head.
 // It walks the request's keys in tiles of 64, staged once through LDS for all four
-// waves: K pages as they lie in the cache ([key, d], rows padded against bank
-// conflicts) and V pages ([d, key]) regrouped so that operand reads are contiguous.  Per wave, per 16-key block:
+// waves (two tiles of LDS: while one is read, the next is written, one barrier a tile):
+// K pages as they lie in the cache ([key, d], rows padded against bank conflicts) and V
+// pages ([d, key]) regrouped so that operand reads are contiguous.  Per wave:
 //
-//   S^T[16 keys, 16 rows]  = K[16 keys, d]   * Q^T[d, 16 rows]        (16x16x32, CT times)
-//   O^T[d, 16 rows]       += V^T[d, 16 keys] * P^T[16 keys, 16 rows]  (16x16x16, CT times)
+//   S^T[16 keys, 16 rows]  = K[16 keys, d]   * Q^T[d, 16 rows]        (16x16x32, per key block)
+//   O^T[d, 16 rows]       += V^T[d, 32 keys] * P^T[32 keys, 16 rows]  (16x16x32, per two key blocks)
 //
-// The accumulator layout of S^T is the B-operand layout of the second product, so the
-// probabilities stay in registers.  Softmax state is float32 per row; the running
-// output is rescaled only when a row's maximum moved by more than 2^8.
+// A lane's four accumulator values of S^T for key blocks a and b are the eight values of
+// the B operand of the second product, if the product's k index 8*quad + e stands for key
+// 4*quad + e of block a (e < 4) or key 4*quad + e - 4 of block b: V is laid out in LDS to
+// match, so the probabilities stay in registers.  Softmax state is float32 per row; the
+// running output is rescaled only when a row's maximum moved by more than 2^8.
 // A key is visible to a row iff first <= key <= the row's position; keys beyond the
 // request's last position and pages given back behind a window are zeroed on their way
 // into LDS, so nothing that was not written by this request reaches a product.
@@ -43,6 +46,11 @@ __device__ __forceinline__ s16x4_t pack_bf16x4(const float* p) {
 constexpr int kWaves = 4;
 constexpr int kKeyBlocks = 4;  // 16-key blocks per LDS tile
 
+template <int D>
+constexpr int tile_bytes() {
+  return kKeyBlocks * 16 * (D + 8) * 2 + kKeyBlocks * D * 16 * 2;  // K rows padded, then V
+}
+
 template <int D, int CT>
 __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
@@ -53,38 +61,50 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   constexpr int NJ = D / 16;
   constexpr int NC = D / 32;
   constexpr int KROW = D + 8;  // padded K row in LDS (elements)
-  __shared__ __attribute__((aligned(16))) bf16_t k_lds[kKeyBlocks * 16 * KROW];
-  __shared__ __attribute__((aligned(16))) bf16_t v_lds[kKeyBlocks * D * 16];
+  constexpr int K_ELEMS = kKeyBlocks * 16 * KROW;
+  constexpr int TILE_ELEMS = tile_bytes<D>() / 2;
+  extern __shared__ __attribute__((aligned(16))) bf16_t tiles[];  // two tiles: [K | V] each
 
   const int g = nh / nkv;
   const int bq = (64 * CT) / g;  // tokens per block
   const int hk = blockIdx.y;
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int col = lane & 15;
   const int quad = lane >> 4;
 
-  // which request and which of its token tiles: tiles are numbered request by request
-  int req = -1, t0 = 0, t_end = 0;
+  // Which request and which two of its token tiles.  Under the causal mask a request's late
+  // tiles see many keys and its early tiles few, so a block takes tile n-1-p and then tile p
+  // (p < n/2; the middle tile of an odd count once): every block of a request then walks
+  // about the same number of key tiles.  Pairs are numbered request by request.
+  int req = -1, pair = 0, n_tiles = 0, q_begin = 0, q_end = 0;
   {
-    // late tiles of a request have the most keys: hand them out first (reverse numbering)
-    int tile = gridDim.x - 1 - blockIdx.x;
+    int idx = blockIdx.x;
     for (int r = 0; r < num_reqs; ++r) {
       const int b = q_start[r], e = q_start[r + 1];
-      const int tiles = (e - b + bq - 1) / bq;
-      if (tile < tiles) {
+      const int tiles_r = (e - b + bq - 1) / bq;
+      const int pairs_r = (tiles_r + 1) / 2;
+      if (idx < pairs_r) {
         req = r;
-        t0 = b + tile * bq;
-        t_end = (t0 + bq < e) ? t0 + bq : e;
+        pair = idx;
+        n_tiles = tiles_r;
+        q_begin = b;
+        q_end = e;
         break;
       }
-      tile -= tiles;
+      idx -= pairs_r;
     }
   }
-  if (req < 0) return;  // the grid is an upper bound on the number of tiles
-  const int n_tok = t_end - t0;
+  if (req < 0) return;  // the grid is an upper bound on the number of pairs
   const int32_t* row_table = table + static_cast<int64_t>(slots[req]) * table_stride;
+  for (int turn = 0; turn < 2; ++turn) {
+  const int tile = (turn == 0) ? n_tiles - 1 - pair : pair;
+  if (turn == 1 && tile == n_tiles - 1 - pair) break;  // the middle tile was the first turn
+  if (turn == 1) __syncthreads();  // the first turn's last tile has been consumed by every wave
+  const int t0 = q_begin + tile * bq;
+  const int t_end = (t0 + bq < q_end) ? t0 + bq : q_end;
+  const int n_tok = t_end - t0;
   const int pos_lo = positions[t0];
   const int pos_hi = positions[t_end - 1];  // positions rise by one along a request's tokens
   const int first_lo = (window > 0 && pos_lo - window + 1 > 0) ? pos_lo - window + 1 : 0;
@@ -114,27 +134,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
       }
     }
   }
-  // wave-uniform bounds of what this wave's rows can see
-  int wave_pos_hi = -1;
-#pragma unroll
-  for (int ct = 0; ct < CT; ++ct) wave_pos_hi = max(wave_pos_hi, my_pos[ct]);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) wave_pos_hi = max(wave_pos_hi, __shfl_xor(wave_pos_hi, o, 64));
-
-  f32x4_t o_acc[CT][NJ];
-  float m[CT], l[CT];
+  // Bounds of what this wave's live rows can see.  They are the same in every lane after
+  // the exchange and are made scalar, so that the conditions on them below are scalar
+  // branches: matrix instructions must be skipped by a branch, never by a lane mask.
+  int wave_pos_hi = -1, wave_pos_lo = 0x7fffffff, wave_first_hi = 0;
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
-    m[ct] = -INFINITY;
-    l[ct] = 0.f;
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) o_acc[ct][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  }
-
-  // wave-uniform bounds of the positions of this wave's live rows
-  int wave_pos_lo = 0x7fffffff, wave_first_hi = 0;
-#pragma unroll
-  for (int ct = 0; ct < CT; ++ct) {
+    wave_pos_hi = max(wave_pos_hi, my_pos[ct]);
     if (live[ct]) {
       wave_pos_lo = min(wave_pos_lo, my_pos[ct]);
       wave_first_hi = max(wave_first_hi, my_first[ct]);
@@ -142,8 +148,22 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
+    wave_pos_hi = max(wave_pos_hi, __shfl_xor(wave_pos_hi, o, 64));
     wave_pos_lo = min(wave_pos_lo, __shfl_xor(wave_pos_lo, o, 64));
     wave_first_hi = max(wave_first_hi, __shfl_xor(wave_first_hi, o, 64));
+  }
+  wave_pos_hi = __builtin_amdgcn_readfirstlane(wave_pos_hi);
+  wave_pos_lo = __builtin_amdgcn_readfirstlane(wave_pos_lo);
+  wave_first_hi = __builtin_amdgcn_readfirstlane(wave_first_hi);
+
+  f32x4_t o_acc[CT][NJ];
+  float m[CT], l[CT];  // m: the reference maximum of the raw (unscaled) scores
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    m[ct] = -INFINITY;
+    l[ct] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) o_acc[ct][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
   const int blocks_per_page = page_size / 16;
@@ -231,15 +251,16 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
       vreg[i] = val;
     }
   };
-
-  fetch_tile(kb_first);
-  for (int kb0 = kb_first; kb0 < kb_end; kb0 += kKeyBlocks) {
-    __syncthreads();  // the previous tile has been consumed
+  // Registers to LDS.  K: [key][KROW].  V: [pair of key blocks][16-row group j][quad][row in
+  // group][8 keys], the eight keys being 4*quad .. +4 of the pair's first block and then of
+  // its second, so that the 64 lanes of an A-operand read (lane = quad*16 + row) touch 1024
+  // consecutive bytes.
+  auto store_tile = [&](int buf) {
+    bf16_t* k_lds = tiles + buf * TILE_ELEMS;
+    bf16_t* v_lds = k_lds + K_ELEMS;
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i)
       *reinterpret_cast<uint4*>(k_lds + (i * ROWS_PER_STEP + k_row0) * KROW + k_piece * 8) = kreg[i];
-    // V in LDS: [key block][16-row group j][quad][row in group][4 keys], so that the 64
-    // lanes of an A-operand read (lane = quad*16 + row) touch 512 consecutive bytes
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
       int kbi, rem;
@@ -252,15 +273,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
       }
       const int drow = rem >> 1;
       const int half = rem & 1;
-      bf16_t* dst = v_lds + (((kbi * NJ + (drow >> 4)) * 4 + 2 * half) * 16 + (drow & 15)) * 4;
+      // keys 8*half .. +4 belong to quad 2*half, the next four to quad 2*half + 1
+      bf16_t* dst = v_lds + (((((kbi >> 1) * NJ + (drow >> 4)) * 4 + 2 * half) * 16 + (drow & 15)) * 8) +
+                    4 * (kbi & 1);
       *reinterpret_cast<uint2*>(dst) = make_uint2(vreg[i].x, vreg[i].y);
-      *reinterpret_cast<uint2*>(dst + 64) = make_uint2(vreg[i].z, vreg[i].w);
+      *reinterpret_cast<uint2*>(dst + 16 * 8) = make_uint2(vreg[i].z, vreg[i].w);
     }
-    __syncthreads();
-    if (kb0 + kKeyBlocks < kb_end) fetch_tile(kb0 + kKeyBlocks);  // in flight while this tile is used
+  };
 
-    // ---- scores of the tile for this wave's rows
-    if (kb0 * 16 > wave_pos_hi) continue;  // nothing here is visible to this wave (uniform)
+  const float unit = 8.f / scale_log2e;  // 2^8 in units of the raw scores
+  auto work_tile = [&](int kb0, int buf) {
+    const bf16_t* k_lds = tiles + buf * TILE_ELEMS;
+    const bf16_t* v_lds = k_lds + K_ELEMS;
+    // ---- raw scores of the tile for this wave's rows
     f32x4_t s[CT][kKeyBlocks];
 #pragma unroll
     for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
@@ -274,16 +299,16 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
 #pragma unroll
         for (int c = 0; c < NC; ++c)
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], qb[ct][c], acc, 0, 0, 0);
-        s[ct][kbi] = acc * scale_log2e;
+        s[ct][kbi] = acc;
       }
     }
     // ---- softmax update per row over the 64 keys of the tile; a tile that every live row of
     // the wave sees whole needs no masks
     const bool whole = (kb0 + kKeyBlocks) * 16 - 1 <= wave_pos_lo && kb0 * 16 >= wave_first_hi;
     // The reference maximum of a row only moves when the tile's maximum exceeds it by more
-    // than 2^8: probabilities then stay below 256, which bfloat16 and the float32 sums hold
-    // easily, and the running output is rescaled rarely instead of at every tile.
-    s16x4_t pb[CT][kKeyBlocks];
+    // than 2^8 (after scaling): probabilities then stay below 256, which bfloat16 and the
+    // float32 sums hold easily, and the running output is rescaled rarely instead of at
+    // every tile.  The scale is applied inside the exponent's multiply-add.
     float mx[CT];
     bool moved = false;
 #pragma unroll
@@ -307,13 +332,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
       v = fmaxf(v, __shfl_xor(v, 16, 64));
       v = fmaxf(v, __shfl_xor(v, 32, 64));
       mx[ct] = v;
-      moved = moved || (v > m[ct] + 8.f);  // also true for the first visible key (m = -inf)
+      moved = moved || (v > m[ct] + unit);  // also true for the first visible key (m = -inf)
     }
     if (__any(moved)) {
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) {
-        if (mx[ct] > m[ct] + 8.f) {
-          const float alpha = __builtin_amdgcn_exp2f(m[ct] - mx[ct]);  // 0 when m was -inf
+        if (mx[ct] > m[ct] + unit) {
+          const float alpha = __builtin_amdgcn_exp2f((m[ct] - mx[ct]) * scale_log2e);  // 0 when m was -inf
           m[ct] = mx[ct];
           l[ct] *= alpha;
 #pragma unroll
@@ -321,36 +346,49 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
         }
       }
     }
+    bf16x8_t pb[CT][kKeyBlocks / 2];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
-      const float m_safe = (m[ct] == -INFINITY) ? 0.f : m[ct];
+      const float neg_mc = (m[ct] == -INFINITY) ? 0.f : -m[ct] * scale_log2e;
       float ps = 0.f;
 #pragma unroll
       for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
-        float p[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          p[i] = __builtin_amdgcn_exp2f(s[ct][kbi][i] - m_safe);
-          ps += p[i];
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ct][kbi][i], scale_log2e, neg_mc));
+          ps += p;
+          pb[ct][kbi >> 1][4 * (kbi & 1) + i] = static_cast<__bf16>(p);
         }
-        pb[ct][kbi] = pack_bf16x4(p);
       }
       ps += __shfl_xor(ps, 16, 64);
       ps += __shfl_xor(ps, 32, 64);
       l[ct] += ps;
     }
-    // ---- O^T += V^T P^T
+    // ---- O^T += V^T P^T, two key blocks a product
 #pragma unroll
-    for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
-      if ((kb0 + kbi) * 16 > wave_pos_hi) break;  // uniform: later blocks weigh nothing
+    for (int pr = 0; pr < kKeyBlocks / 2; ++pr) {
+      if ((kb0 + 2 * pr) * 16 > wave_pos_hi) break;  // scalar: later blocks weigh nothing
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const s16x4_t va = *reinterpret_cast<const s16x4_t*>(v_lds + (((kbi * NJ + j) * 4 + quad) * 16 + col) * 4);
+        const bf16x8_t va =
+            *reinterpret_cast<const bf16x8_t*>(v_lds + (((pr * NJ + j) * 4 + quad) * 16 + col) * 8);
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
-          o_acc[ct][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb[ct][kbi], o_acc[ct][j], 0, 0, 0);
+          o_acc[ct][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[ct][pr], o_acc[ct][j], 0, 0, 0);
       }
     }
+  };
+
+  fetch_tile(kb_first);
+  store_tile(0);
+  __syncthreads();
+  int buf = 0;
+  for (int kb0 = kb_first; kb0 < kb_end; kb0 += kKeyBlocks, buf ^= 1) {
+    const bool more = kb0 + kKeyBlocks < kb_end;
+    if (more) fetch_tile(kb0 + kKeyBlocks);  // in flight while this tile is used
+    if (kb0 * 16 <= wave_pos_hi) work_tile(kb0, buf);  // scalar: else nothing here is visible to this wave
+    if (more) store_tile(buf ^ 1);
+    __syncthreads();  // the next tile is whole, and this one has been consumed
   }
 
 #pragma unroll
@@ -365,6 +403,28 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
       *reinterpret_cast<s16x4_t*>(op + 16 * j) = pack_bf16x4(vv);
     }
   }
+  }  // turn
+}
+
+template <int D, int CT>
+int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t* k_cache,
+                      const bf16_t* v_cache, const int32_t* table, int table_stride,
+                      const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
+                      int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
+                      hipStream_t stream) {
+  const int g = nh / nkv;
+  const int bq = (64 * CT) / g;
+  // every request may end in a ragged tile and have an odd number of tiles
+  const int max_pairs = ((T + bq - 1) / bq + R) / 2 + R;
+  constexpr int lds_bytes = 2 * tile_bytes<D>();
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&prefill_attention_kernel<D, CT>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  if (attr != hipSuccess) return kvc_fail("kvc_prefill_attention: the kernel's LDS size was refused");
+  hipLaunchKernelGGL((prefill_attention_kernel<D, CT>), dim3(max_pairs, nkv), dim3(kWaves * 64),
+                     lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
+                     q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window);
+  return kvc_check_launch("kvc_prefill_attention");
 }
 
 template <int D>
@@ -374,13 +434,17 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
                    int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
                    hipStream_t stream) {
   const int g = nh / nkv;
-  constexpr int CT = 2;
-  const int bq = (64 * CT) / g;
-  const int max_tiles = (T + bq - 1) / bq + R;  // every request may end in a ragged tile
-  hipLaunchKernelGGL((prefill_attention_kernel<D, CT>), dim3(max_tiles, nkv), dim3(kWaves * 64), 0,
-                     stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
-                     q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window);
-  return kvc_check_launch("kvc_prefill_attention");
+  // Tiles of 128 query rows stage each key tile for twice the rows, tiles of 64 make twice
+  // the blocks: the larger ones once their pairs alone give every compute unit two blocks.
+  const int bq2 = 128 / g > 0 ? 128 / g : 1;
+  const int64_t pairs2 = static_cast<int64_t>(((T + bq2 - 1) / bq2 + 1) / 2) * nkv;
+  if (pairs2 >= 512 || g > 64)
+    return launch_prefill_ct<D, 2>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
+                                   q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window,
+                                   stream);
+  return launch_prefill_ct<D, 1>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
+                                 q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window,
+                                 stream);
 }
 
 }  // namespace
@@ -404,6 +468,7 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
                     "most 64 query heads per kv head, page size a multiple of 16)");
   if (T < 0 || R <= 0 || nkv > 65535 || table_stride <= 0 || num_pages <= 0)
     return kvc_fail("kvc_prefill_attention: bad sizes");
+  if (!(scale > 0.f)) return kvc_fail("kvc_prefill_attention: the scale must be positive");
   if (q_stride % 8) return kvc_fail("kvc_prefill_attention: q rows must be 16-byte aligned");
   if (T == 0) return 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);

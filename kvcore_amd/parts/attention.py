@@ -122,7 +122,7 @@ class PagedAttention(Mixer):
             ops.rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim,
                               interleaved=interleaved, kv_slot=kv_slot, nh=self.num_heads,
                               nkv=self.num_kv_heads, d=self.head_dim, write_kv=call.write_cache)
-            if ctx.max_query_len > 1 and ops.prefill_attention_supported(
+            if ctx.max_query_len > 1 and self.scale > 0 and ops.prefill_attention_supported(
                     self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
                 # portions of prompts (single tokens may ride along): tiles of query rows per block
                 ops.prefill_attention(attn, qkv, k_cache, v_cache, table=group.table,
