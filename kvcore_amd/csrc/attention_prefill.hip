@@ -183,6 +183,16 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   constexpr int ROWS_PER_STEP = 256 / PIECES;  // K rows that the block fetches per step
   const int k_row0 = tid / PIECES;             // this thread's K row within a step
   const int k_piece = tid % PIECES;
+  // element offsets of this thread's pieces within a key block's K rows and V rows
+  int k_off[K_PER_THREAD], v_off[V_PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < K_PER_THREAD; ++i)
+    k_off[i] = ((i * ROWS_PER_STEP + k_row0) & 15) * D + k_piece * 8;
+#pragma unroll
+  for (int i = 0; i < V_PER_THREAD; ++i) {
+    const int rem = (D == 128) ? tid : (tid & 127);
+    v_off[i] = (rem >> 1) * page_size + (rem & 1) * 8;
+  }
   auto fetch_tile = [&](int kb0) {
     const bool tail = (kb0 + kKeyBlocks) * 16 > pos_hi + 1;  // uniform: some keys are not the request's
     int64_t kpage[kKeyBlocks], vpage[kKeyBlocks];  // element offsets of the key blocks, or -1
@@ -191,13 +201,39 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
       const int kb = kb0 + kbi;
       kpage[kbi] = vpage[kbi] = -1;
       if (kb < kb_end) {
-        const int page = row_table[kb / blocks_per_page];
+        const int page = __builtin_amdgcn_readfirstlane(row_table[kb / blocks_per_page]);
         if (page > 0 && page < num_pages) {
           const int sub = kb % blocks_per_page;
           kpage[kbi] = ((static_cast<int64_t>(page) * nkv + hk) * page_size + sub * 16) * D;
           vpage[kbi] = (static_cast<int64_t>(page) * nkv + hk) * D * page_size + sub * 16;
         }
       }
+    }
+    if (!tail) {
+      // every key of the tile is the request's: a scalar base and a fixed offset per piece
+#pragma unroll
+      for (int i = 0; i < K_PER_THREAD; ++i) {
+        int64_t base;
+        if constexpr (ROWS_PER_STEP == 16) {
+          base = kpage[i];
+        } else {
+          base = (k_row0 < 16) ? kpage[2 * i] : kpage[2 * i + 1];
+        }
+        kreg[i] = (base >= 0) ? *reinterpret_cast<const uint4*>(k_cache + base + k_off[i])
+                              : make_uint4(0u, 0u, 0u, 0u);
+      }
+#pragma unroll
+      for (int i = 0; i < V_PER_THREAD; ++i) {
+        int64_t base;
+        if constexpr (D == 128) {
+          base = vpage[i];
+        } else {
+          base = (tid < 128) ? vpage[2 * i] : vpage[2 * i + 1];
+        }
+        vreg[i] = (base >= 0) ? *reinterpret_cast<const uint4*>(v_cache + base + v_off[i])
+                              : make_uint4(0u, 0u, 0u, 0u);
+      }
+      return;
     }
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
@@ -210,23 +246,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
         base = (k_row0 < 16) ? kpage[2 * i] : kpage[2 * i + 1];
       }
       uint4 val = make_uint4(0u, 0u, 0u, 0u);
-      if (base >= 0 && (!tail || kb0 * 16 + key_row <= pos_hi))
-        val = *reinterpret_cast<const uint4*>(k_cache + base + (key_row & 15) * D + k_piece * 8);
+      if (base >= 0 && kb0 * 16 + key_row <= pos_hi)
+        val = *reinterpret_cast<const uint4*>(k_cache + base + k_off[i]);
       kreg[i] = val;
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
       // piece (i*256 + tid) of the tile: key block, then row of the head, then half of 16 keys
-      int kbi, rem;
-      if constexpr (D == 128) {
-        kbi = i;
-        rem = tid;
-      } else {
-        kbi = 2 * i + (tid >> 7);
-        rem = tid & 127;
-      }
-      const int drow = rem >> 1;
-      const int half = rem & 1;
+      const int kbi = (D == 128) ? i : 2 * i + (tid >> 7);
+      const int half = tid & 1;
       int64_t base;
       if constexpr (D == 128) {
         base = vpage[i];
@@ -235,17 +263,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
       }
       uint4 val = make_uint4(0u, 0u, 0u, 0u);
       const int key0 = (kb0 + kbi) * 16 + half * 8;
-      if (base >= 0 && (!tail || key0 <= pos_hi)) {
-        val = *reinterpret_cast<const uint4*>(v_cache + base + static_cast<int64_t>(drow) * page_size + half * 8);
-        if (tail) {
-          const int n_ok = pos_hi - key0 + 1;  // keys key0 .. key0+7 beyond pos_hi are not this request's
-          if (n_ok < 8) {
-            uint32_t w[4] = {val.x, val.y, val.z, val.w};
+      if (base >= 0 && key0 <= pos_hi) {
+        val = *reinterpret_cast<const uint4*>(v_cache + base + v_off[i]);
+        const int n_ok = pos_hi - key0 + 1;  // keys key0 .. key0+7 beyond pos_hi are not this request's
+        if (n_ok < 8) {
+          uint32_t w[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (e >= n_ok) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
-            val = make_uint4(w[0], w[1], w[2], w[3]);
-          }
+          for (int e = 0; e < 8; ++e)
+            if (e >= n_ok) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+          val = make_uint4(w[0], w[1], w[2], w[3]);
         }
       }
       vreg[i] = val;
