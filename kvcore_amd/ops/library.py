@@ -430,10 +430,11 @@ def linear(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tens
     N = w.shape[0]
     skinny_ok = _skinny_operands_ok(x, w)
     # measured on MI355X (N x K of 4096..128256 x 4096..14336): the weight-streaming kernel
-    # wins up to 8 rows everywhere and up to 16 rows unless K or N is very large; it is also
-    # the only one that stores float32
+    # wins up to 8 rows everywhere, up to 16 rows unless K or N is very large and up to 32 rows
+    # for small matrices; it is also the only one that stores float32
     if skinny_ok and (out.dtype == torch.float32 or M <= 8
-                      or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)):
+                      or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)
+                      or (M <= 32 and K <= 4096 and N <= 4096)):
         gemm_skinny_bf16(out, x, w, bias)
         return
     if out.dtype != torch.bfloat16:
