@@ -38,11 +38,13 @@ class _RequestPages:
 
 
 class KVManager:
-    def __init__(self, groups: list[GroupConfig], *, max_num_seqs: int, max_model_len: int) -> None:
+    def __init__(self, groups: list[GroupConfig], *, max_num_seqs: int, max_model_len: int,
+                 shuffle_seed: int | None = None) -> None:
         if max_model_len <= 0:
             raise ValueError("max_model_len must be positive")
         self.groups = list(groups)
-        self.pools = [PagePool(g.num_pages) for g in self.groups]
+        self.pools = [PagePool(g.num_pages, None if shuffle_seed is None else shuffle_seed + i)
+                      for i, g in enumerate(self.groups)]
         self.slots = SlotPool(max_num_seqs)
         self.max_model_len = max_model_len
         self._req_pages: dict[str, list[_RequestPages]] = {}

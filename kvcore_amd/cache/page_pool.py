@@ -9,16 +9,23 @@ free before it.  The reference links block objects; ids in a deque give the same
 
 from __future__ import annotations
 
+import random
 from collections import deque
 from typing import Iterable
 
 
 class PagePool:
-    def __init__(self, num_pages: int) -> None:
+    """``shuffle_seed`` (a debugging aid) starts the free queue in a seeded random order
+    instead of 1, 2, 3, ...: results must not depend on which pages a request gets."""
+
+    def __init__(self, num_pages: int, shuffle_seed: int | None = None) -> None:
         if num_pages < 2:
             raise ValueError(f"a pool needs the null page and at least one more, got {num_pages}")
         self.num_pages = num_pages
-        self._free: deque[int] = deque(range(1, num_pages))
+        order = list(range(1, num_pages))
+        if shuffle_seed is not None:
+            random.Random(shuffle_seed).shuffle(order)
+        self._free: deque[int] = deque(order)
         self._held = bytearray(num_pages)  # 1 while a request holds the page
 
     @property

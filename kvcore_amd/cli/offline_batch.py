@@ -3,7 +3,10 @@
 Reference: scripts/run_llm_engine_offline_batch.py:127-271: the option names and
 meanings it has are kept (``--model --device --block-size --max-model-len
 --max-num-seqs --max-num-scheduled-tokens --max-num-partial-prefills
---max-long-partial-prefills --long-prefill-token-threshold --log-level --log-file``),
+--max-long-partial-prefills --long-prefill-token-threshold --attn-backend
+--local-files-only --log-level --log-file``; ``--revision`` and ``--trust-remote-code``
+are recognised and refused or ignored, since models are local folders and no code of
+theirs is ever run),
 as are its output sections (run metadata, request summary, outputs, timing summary).
 Its hard-coded chat requests are not: requests come from ``--requests FILE`` (a JSON
 list of ``{"request_id", "messages" | "prompt_token_ids", "max_tokens", "temperature",
@@ -26,6 +29,13 @@ def parse_args(argv=None) -> argparse.Namespace:
     p = argparse.ArgumentParser(description="Run offline batch generation through LLMEngine.")
     p.add_argument("--model", required=True, help="model folder (config.json, *.safetensors)")
     p.add_argument("--device", default="cuda:0")
+    p.add_argument("--attn-backend", default=None, choices=["hip"],
+                   help="Attention backend override. Defaults to KVCoreConfig auto selection.")
+    p.add_argument("--revision", default=None, help="not supported: models are local folders")
+    p.add_argument("--trust-remote-code", action="store_true",
+                   help="accepted and ignored: no code from a model folder is ever run")
+    p.add_argument("--local-files-only", action=argparse.BooleanOptionalAction, default=True,
+                   help="models are always read from local folders; --no-local-files-only is refused")
     p.add_argument("--dtype", default=None, choices=[None, "bfloat16", "bf16", "float32", "fp32"])
     p.add_argument("--block-size", type=int, default=16)
     p.add_argument("--max-model-len", type=int, default=None)
@@ -51,7 +61,11 @@ def parse_args(argv=None) -> argparse.Namespace:
     p.add_argument("--log-file", default=None,
                    help="Path for teeing terminal output. Defaults to logs/<script>_<timestamp>.log.")
     p.add_argument("--no-log-file", action="store_true", help="do not tee to a file")
-    return p.parse_args(argv)
+    args = p.parse_args(argv)
+    if args.revision is not None or not args.local_files_only:
+        p.error("models are read from local folders only: --revision and --no-local-files-only "
+                "have no meaning here")
+    return args
 
 
 class _Tee:
@@ -89,7 +103,7 @@ def build_config(args: argparse.Namespace):
 
     return KVCoreConfig(
         model_config=ModelConfig(model=str(Path(args.model).expanduser()), dtype=args.dtype,
-                                 max_model_len=args.max_model_len),
+                                 max_model_len=args.max_model_len, attn_backend=args.attn_backend),
         load_config=LoadConfig(load_format="random" if args.random_weights else "safetensors",
                                seed=args.seed),
         cache_config=CacheConfig(block_size=args.block_size, num_gpu_blocks=args.num_gpu_blocks,
@@ -164,7 +178,11 @@ def main(argv=None) -> int:
         print(f"max_num_scheduled_tokens={args.max_num_scheduled_tokens}")
 
         engine_start = time.perf_counter()
-        engine = LLMEngine(build_config(args))
+        config = build_config(args)
+        print(f"attn_backend={config.model_config.attn_backend}")
+        if args.trust_remote_code:
+            print("trust_remote_code is ignored: no code from a model folder is ever run")
+        engine = LLMEngine(config)
         engine_elapsed = time.perf_counter() - engine_start
         print(f"engine_init_sec={engine_elapsed:.3f}")
         print(f"num_gpu_blocks={engine.engine_core.num_pages}")

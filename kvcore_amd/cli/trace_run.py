@@ -35,6 +35,10 @@ def parse_args(argv=None) -> argparse.Namespace:
     p.add_argument("--device", default="cuda:0")
     p.add_argument("--poison-cache", action="store_true",
                    help="fill the cache with NaN first, so a read of a slot nobody wrote shows")
+    p.add_argument("--shuffle-pages", type=int, default=None, metavar="SEED",
+                   help="hand pages out in a seeded random order (the logits must not change)")
+    p.add_argument("--show-pages", action="store_true",
+                   help="print each step's page ids per request on standard error")
     return p.parse_args(argv)
 
 
@@ -59,7 +63,7 @@ def main(argv=None) -> int:
     out_dir.mkdir(parents=True, exist_ok=True)
     session = TraceSession(args.model, dtype, max_tokens=args.max_tokens, block_size=args.block_size,
                            max_num_seqs=args.max_num_seqs, device=args.device,
-                           poison_cache=args.poison_cache)
+                           poison_cache=args.poison_cache, shuffle_pages=args.shuffle_pages)
     print("trace_run: ready", file=sys.stderr, flush=True)
 
     for line in sys.stdin:
@@ -67,7 +71,13 @@ def main(argv=None) -> int:
         if not line:
             continue
         record = json.loads(line)
+        if args.show_pages:
+            live_before = {str(item["id"]) for item in record.get("entries", [])}
         out = session.run_step(record)
+        if args.show_pages:
+            pages = {rid: session.manager.page_ids(rid) for rid in sorted(live_before)
+                     if session.manager.is_admitted(rid)}
+            print(f"pages {record['step']} {json.dumps(pages)}", file=sys.stderr, flush=True)
         if out is not None and out.logits is not None:
             host = out.logits.detach().to("cpu", torch.float32).numpy()
             np.ascontiguousarray(host, dtype="<f4").tofile(out_dir / f"{record['step']}.f32")

@@ -18,6 +18,11 @@ DTYPE_NAMES = {
 }
 
 
+# The reference chooses between "torch_paged" and "triton_paged" (config.py:28, 170-178);
+# here the paged attention is always the HIP kernels.
+ATTN_BACKENDS = ("hip",)
+
+
 def canonical_dtype(name: str | None) -> str | None:
     """``"bfloat16"`` or ``"float32"`` from any of their usual spellings."""
     if name is None:
@@ -37,10 +42,15 @@ class ModelConfig:
     tokenizer: str | Path | None = None
     dtype: str | None = None
     max_model_len: int | None = None
+    attn_backend: str | None = None
 
     def __post_init__(self) -> None:
         if self.max_model_len is not None and self.max_model_len <= 0:
             raise ValueError(f"max_model_len must be positive, got {self.max_model_len}")
+        if self.attn_backend not in (None, *ATTN_BACKENDS):
+            raise ValueError(
+                f"unsupported attn_backend {self.attn_backend!r}; this engine has one attention "
+                f"backend: {', '.join(ATTN_BACKENDS)} (the HIP kernels for gfx950)")
         object.__setattr__(self, "dtype", canonical_dtype(self.dtype))
 
 
@@ -121,3 +131,8 @@ class KVCoreConfig:
     cache_config: CacheConfig = field(default_factory=CacheConfig)
     scheduler_config: SchedulerConfig = field(default_factory=SchedulerConfig)
     device_config: DeviceConfig = field(default_factory=DeviceConfig)
+
+    def __post_init__(self) -> None:
+        # an unset attention backend is filled in, as the reference does (config.py:170-192)
+        if self.model_config.attn_backend is None:
+            object.__setattr__(self.model_config, "attn_backend", ATTN_BACKENDS[0])

@@ -19,14 +19,15 @@ from .runner import ModelRunner, StepEntry, StepOutput, build_model
 class TraceSession:
     def __init__(self, model_dir: str, dtype: torch.dtype, *, max_tokens: int, block_size: int = 16,
                  max_num_seqs: int = 8, device: str = "cuda:0", poison_cache: bool = False,
-                 model=None) -> None:
+                 shuffle_pages: int | None = None, model=None) -> None:
         self.model = model if model is not None else build_model(model_dir, dtype, device)
         page = block_size
         capacity = -(-max_tokens // 64) * 64
         self.capacity = capacity
         self.num_pages = -(-capacity // page) + 1  # + the null page
         groups = [GroupConfig(page, self.num_pages, g.need.window) for g in self.model.cache_groups]
-        self.manager = KVManager(groups, max_num_seqs=max_num_seqs, max_model_len=capacity)
+        self.manager = KVManager(groups, max_num_seqs=max_num_seqs, max_model_len=capacity,
+                                 shuffle_seed=shuffle_pages)
         self.runner = ModelRunner(self.model, page_size=page, num_pages=self.num_pages,
                                   max_num_seqs=max_num_seqs, max_num_tokens=capacity,
                                   max_model_len=capacity)

@@ -21,6 +21,15 @@ def test_pool_reserves_the_null_page_and_hands_out_in_order():
     pool.check()
 
 
+def test_a_shuffled_pool_hands_out_every_page_once_in_another_order():
+    plain_order = PagePool(40).take(39)
+    shuffled = PagePool(40, shuffle_seed=1)
+    order = shuffled.take(39)
+    assert sorted(order) == plain_order == list(range(1, 40)) and order != plain_order
+    assert PagePool(40, shuffle_seed=1).take(39) == order  # the seed fixes the order
+    shuffled.check()
+
+
 def test_pool_refuses_double_free_overdraw_and_foreign_ids():
     pool = PagePool(4)
     pages = pool.take(2)

@@ -106,5 +106,10 @@ def test_engine_config_validation():
         SchedulerConfig(long_prefill_token_threshold=-1)
     cfg = KVCoreConfig(ModelConfig(model="x", dtype="bf16"))
     assert cfg.model_config.dtype == "bfloat16"
+    # the attention backend is filled in when unset (config.py:170-192); the reference's own
+    # backends are refused by name
+    assert ModelConfig(model="x").attn_backend is None and cfg.model_config.attn_backend == "hip"
+    with pytest.raises(ValueError, match="hip"):
+        ModelConfig(model="x", attn_backend="triton_paged")
     assert (cfg.cache_config.block_size, cfg.scheduler_config.max_num_seqs,
             cfg.scheduler_config.max_num_scheduled_tokens) == (16, 8, 512)

@@ -204,6 +204,33 @@ def test_mixed_batches_with_page_reuse(models, name, dtype):
     assert session.manager.num_free_pages()[0] == session.num_pages - 1
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
+def test_logits_do_not_depend_on_which_pages_are_used(models, dtype):
+    """The mixed trace again with the free pages handed out in a shuffled order: the same
+    bits at every position, since only the place in the cache changes, not the arithmetic."""
+    folder, cfg, weights, page = models["D"]
+    base = PROMPT_LENS["D"]
+    lens = base + [n + 3 for n in base]
+    token_lists = {f"q{i}": random_tokens(n + EXTRA, cfg["vocab_size"], seed=600 + i) for i, n in enumerate(lens)}
+    rounded = sorted((-(-len(t) // 64) * 64 for t in token_lists.values()), reverse=True)
+    steps = mixed_trace(token_lists, seed=9)
+    results, orders = [], []
+    for shuffle in (None, 3):
+        session = session_for(folder, dtype, page, max_tokens=sum(rounded[:4]), shuffle_pages=shuffle)
+        got, starts, first_pages = {}, {}, []
+        for rec in steps:
+            got.update(collect_one(session, rec, starts))
+            if not first_pages:
+                first_pages = [p for rid in session.manager.live_requests()
+                               for p in session.manager.page_ids(rid)[0]]
+        results.append(got)
+        orders.append(first_pages)
+    assert orders[0] != orders[1], "the shuffle did not change the pages"
+    assert results[0].keys() == results[1].keys()
+    for key, row in results[0].items():
+        assert torch.equal(row, results[1][key]), key
+
+
 def collect_one(session, rec, starts):
     got = {}
     offsets = {item["id"]: starts.get(item["id"], 0) for item in rec["entries"]}
