@@ -65,13 +65,16 @@ class DecoderModel:
         self._owned: list[tuple[str, Part]] = [(spec.embed_prefix, self.embed),
                                                (spec.final_norm_prefix, self.final_norm),
                                                (spec.head_prefix, self.head)]
+        if spec.position_prefixes and len(spec.position_prefixes) != len(self.positions):
+            raise ValueError("position_prefixes must name every position encoding")
+        for i, pe in enumerate(self.positions):
+            prefix = spec.position_prefixes[i] if spec.position_prefixes else f"model.positions.{i}"
+            self._owned.append((prefix, pe))
         for layer, block in zip(spec.layers, self.blocks):
             for sub, part in block.children().items():
                 self._owned.append((f"{layer.prefix}.{sub}", part))
         for _, part in self._owned:
             part.setup(self.runtime)
-        for pe in self.positions:
-            pe.setup(self.runtime)
 
         self._plan_caches()
         self.params: dict[str, BoundParam] = {}
@@ -153,7 +156,7 @@ class DecoderModel:
     def graph_safe(self) -> bool:
         """True iff every part says its forward may be captured into a HIP graph (it reads
         nothing from the device and decides nothing on the host per step)."""
-        owned = [part for _, part in self._owned] + list(self.positions) + list(self.blocks)
+        owned = [part for _, part in self._owned] + list(self.blocks)
         return all(getattr(part, "graph_safe", True) for part in owned)
 
     def num_param_bytes(self) -> int:

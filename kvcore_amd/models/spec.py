@@ -42,6 +42,9 @@ class ModelSpec:
     schedule: tuple[ScheduleEntry, ...] = ()
     tie_word_embeddings: bool = False
     eos_token_ids: tuple[int, ...] = ()
+    # checkpoint prefixes of the position encodings' own parameters, one per entry of
+    # ``positions`` (empty: "model.positions.<i>"; a rotary encoding has no parameters)
+    position_prefixes: tuple[str, ...] = ()
     embed_prefix: str = "model.embed_tokens"
     final_norm_prefix: str = "model.norm"
     head_prefix: str = "lm_head"

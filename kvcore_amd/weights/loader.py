@@ -153,6 +153,9 @@ def checkpoint_layout(model_spec) -> dict[str, tuple[tuple[int, ...], str, str]]
                                             hidden_size=model_spec.hidden_size,
                                             tied=model_spec.tie_word_embeddings)),
     ]
+    for i, ps in enumerate(model_spec.positions):
+        prefix = model_spec.position_prefixes[i] if model_spec.position_prefixes else f"model.positions.{i}"
+        owned.append((prefix, parts.POSITION_ENCODINGS.build(ps)))
     for layer in model_spec.layers:
         mixer = parts.MIXERS.build(layer.mixer, position=None)
         ffn = parts.FEED_FORWARDS.build(layer.ffn)
