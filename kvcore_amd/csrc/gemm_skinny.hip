@@ -15,6 +15,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
 #include <cstdlib>
 
 #include "device_utils.h"
@@ -56,13 +57,35 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v, int n_left)
   }
 }
 
+// Optional work around the product, all of it by the wave that holds the finished sums:
+//  - in_ss: the rows of A are activations not yet normalised (a gain is already applied);
+//    row m's products are multiplied by rsqrt(sum_p in_ss[m][p] / in_width + in_eps), which
+//    is what normalising the row first would have given;
+//  - residual: the product (+ bias) is added into the float32 residual stream, C receives
+//    bfloat16(residual * gain) and out_ss[m][block] the sum of squares of the new residual
+//    over this block's columns: the next product's in_ss.
+struct SkinnyExtras {
+  const float* in_ss;
+  int in_parts;
+  float in_width;
+  float in_eps;
+  float* residual;
+  int64_t ldr;
+  const float* gain;
+  float* out_ss;
+};
+
 // GATED: the two row tiles of a wave are rows n of the first N weight rows (gate) and rows
 // N + n (up), and the stored value is silu(gate) * up, each factor rounded to bfloat16
 // first as if it had been stored.
-template <int RT, int NT, int U, int MAXW, typename OutT, bool GATED>
+// FOLD: bit 0, the rows of A carry a scale factor still to be applied (ex.in_ss); bit 1, the
+// result goes into the residual stream (ex.residual).  Kernels without these keep their
+// register count, on which the number of waves in flight depends.
+template <int RT, int NT, int U, int MAXW, typename OutT, bool GATED, int FOLD = 0>
 __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restrict__ A,
                                    const bf16_t* __restrict__ W, const bf16_t* __restrict__ bias,
-                                   int M, int N, int K, int64_t lda, int64_t ldc, int k_per_wave) {
+                                   int M, int N, int K, int64_t lda, int64_t ldc, int k_per_wave,
+                                   const SkinnyExtras ex) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
   extern __shared__ float red[];  // [waves - 1][RT * NT][64][4]
   // wave-uniform values are made scalar on purpose: a condition on them becomes a scalar
@@ -97,6 +120,10 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  float row_scale[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) row_scale[nt] = 1.f;
 
   // Whole steps of 64 along K first, software-pipelined: the loads of the next STAGES - 1
   // steps are in flight while a step is multiplied (a lane reads 2 x 16 bytes = a row reads
@@ -135,6 +162,47 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
 #pragma unroll
   for (int st = 0; st < STAGES - 1; ++st)
     if (st < n64) load_step(st, st);
+  // The rows' scale factors, worked out by the wave that will need them at the end while its
+  // first weight loads are on their way, four tokens at a time (more would cost registers and
+  // with them waves in flight).  Token by token the wave reads the row's parts (four a lane)
+  // and adds them up in the fixed order of a butterfly, so the result does not depend on
+  // anything but the parts.
+  if ((FOLD & 1) && wave == 0) {
+    const bool vec = (ex.in_parts % 4 == 0) && ((reinterpret_cast<uintptr_t>(ex.in_ss) & 15) == 0);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int n_tok = (M - nt * 16 < 16) ? M - nt * 16 : 16;  // scalar
+      // all loads of a batch first, then its sums
+      float mine = 0.f;
+      for (int t0 = 0; t0 < n_tok; t0 += 4) {
+        float part[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          part[i] = 0.f;
+          if (t0 + i < n_tok) {
+            const float* parts = ex.in_ss + static_cast<int64_t>(nt * 16 + t0 + i) * ex.in_parts;
+            if (vec) {
+              for (int p = 4 * lane; p < ex.in_parts; p += 256) {
+                const f32x4_t v = *reinterpret_cast<const f32x4_t*>(parts + p);
+                part[i] += (v[0] + v[1]) + (v[2] + v[3]);
+              }
+            } else {
+              for (int p = lane; p < ex.in_parts; p += 64) part[i] += parts[p];
+            }
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (t0 + i < n_tok) {
+            const float total = wave_sum(part[i]);
+            if (col == t0 + i) mine = total;
+          }
+        }
+      }
+      row_scale[nt] = rsqrtf(mine / ex.in_width + ex.in_eps);
+    }
+  }
+
   for (int i = 0; i < n64; i += STAGES) {
 #pragma unroll
     for (int j = 0; j < STAGES; ++j) {
@@ -212,11 +280,57 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
       f32x4_t y;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float gv = to_float(from_float<bf16_t>(acc[0][nt][i] + bg[i]));
-        const float uv = to_float(from_float<bf16_t>(acc[1][nt][i] + bu[i]));
+        const float gv = to_float(from_float<bf16_t>(acc[0][nt][i] * row_scale[nt] + bg[i]));
+        const float uv = to_float(from_float<bf16_t>(acc[1][nt][i] * row_scale[nt] + bu[i]));
         y[i] = gv / (1.f + expf(-gv)) * uv;
       }
       store4<OutT>(C + static_cast<int64_t>(tok) * ldc + n_first, y, n_left);
+    }
+    return;
+  }
+  if constexpr ((FOLD & 2) != 0 && sizeof(OutT) == 2) {
+    {
+      float ss[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) ss[nt] = 0.f;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int n_first = n0 + rt * 16 + 4 * quad;
+        const int n_left = N - n_first;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const int tok = nt * 16 + col;
+          if (tok >= M || n_left <= 0) continue;
+          float* rp = ex.residual + static_cast<int64_t>(tok) * ex.ldr + n_first;
+          bf16_t* cp = reinterpret_cast<bf16_t*>(C) + static_cast<int64_t>(tok) * ldc + n_first;
+          if (n_left >= 4 && ((reinterpret_cast<uintptr_t>(rp) | reinterpret_cast<uintptr_t>(ex.gain + n_first)) & 15) == 0 &&
+              (reinterpret_cast<uintptr_t>(cp) & 7) == 0) {
+            f32x4_t b = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            if (bias != nullptr)
+              for (int i = 0; i < 4; ++i) b[i] = to_float(bias[n_first + i]);
+            const f32x4_t r = *reinterpret_cast<const f32x4_t*>(rp) + (acc[rt][nt] * row_scale[nt] + b);
+            *reinterpret_cast<f32x4_t*>(rp) = r;
+            store4<bf16_t>(cp, r * *reinterpret_cast<const f32x4_t*>(ex.gain + n_first), 4);
+            ss[nt] += (r[0] * r[0] + r[1] * r[1]) + (r[2] * r[2] + r[3] * r[3]);
+          } else {
+            for (int i = 0; i < 4 && i < n_left; ++i) {
+              const float b = (bias != nullptr) ? to_float(bias[n_first + i]) : 0.f;
+              const float r = rp[i] + (acc[rt][nt][i] * row_scale[nt] + b);
+              rp[i] = r;
+              cp[i] = from_float<bf16_t>(r * ex.gain[n_first + i]);
+              ss[nt] += r * r;
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        float v = ss[nt];
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        const int tok = nt * 16 + col;
+        if (quad == 0 && tok < M) ex.out_ss[static_cast<int64_t>(tok) * gridDim.x + blockIdx.x] = v;
+      }
     }
     return;
   }
@@ -232,22 +346,36 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
     for (int nt = 0; nt < NT; ++nt) {
       const int tok = nt * 16 + col;
       if (tok >= M) continue;
-      store4<OutT>(C + static_cast<int64_t>(tok) * ldc + n_first, acc[rt][nt] + bv, n_left);
+      store4<OutT>(C + static_cast<int64_t>(tok) * ldc + n_first, acc[rt][nt] * row_scale[nt] + bv, n_left);
     }
   }
 }
 
 template <int RT, int NT, typename OutT, bool GATED = false>
 void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
-            int64_t lda, int64_t ldc, int waves, int k_per_wave, hipStream_t stream) {
+            int64_t lda, int64_t ldc, int waves, int k_per_wave, const SkinnyExtras& ex,
+            hipStream_t stream) {
   // steps in flight by what fits in registers beside the accumulators
   constexpr int STAGES = (RT + NT <= 5) ? 4 : ((RT + NT <= 6) ? 3 : 2);
   constexpr int MAXW = (RT >= 2) ? 4 : 8;
   const size_t lds = static_cast<size_t>(waves - 1) * RT * NT * 64 * 4 * sizeof(float);
   const int rows_per_block = GATED ? 16 : 16 * RT;
-  hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, STAGES, MAXW, OutT, GATED>),
-                     dim3((N + rows_per_block - 1) / rows_per_block), dim3(waves * 64), lds, stream,
-                     C, A, W, bias, M, N, K, lda, ldc, k_per_wave);
+  const dim3 grid((N + rows_per_block - 1) / rows_per_block), block(waves * 64);
+  const int fold = (ex.in_ss != nullptr ? 1 : 0) | (ex.residual != nullptr ? 2 : 0);
+#define KVC_SKINNY_LAUNCH(FOLD_)                                                                   \
+  hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, STAGES, MAXW, OutT, GATED, FOLD_>), grid, block, \
+                     lds, stream, C, A, W, bias, M, N, K, lda, ldc, k_per_wave, ex)
+  if constexpr (NT == 1 && sizeof(OutT) == 2) {  // folded norms are for steps of few rows
+    switch (fold) {
+      case 0: KVC_SKINNY_LAUNCH(0); break;
+      case 1: KVC_SKINNY_LAUNCH(1); break;
+      case 2: if constexpr (!GATED) KVC_SKINNY_LAUNCH(2); break;
+      default: if constexpr (!GATED) KVC_SKINNY_LAUNCH(3); break;
+    }
+  } else {
+    KVC_SKINNY_LAUNCH(0);
+  }
+#undef KVC_SKINNY_LAUNCH
 }
 
 // The launch shape is a function of N and K alone, so that a row's sums do not depend on
@@ -276,14 +404,14 @@ inline void pick_shape(int N, int K, int* rt_out, int* waves_out) {
 
 template <typename OutT>
 int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
-             int64_t lda, int64_t ldc, hipStream_t stream) {
+             int64_t lda, int64_t ldc, const SkinnyExtras& ex, hipStream_t stream) {
   int rt, waves;
   pick_shape(N, K, &rt, &waves);
   const int nt = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 63) / 64 * 64;
 #define KVC_SKINNY(RT_, NT_) \
-  launch<RT_, NT_, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream)
+  launch<RT_, NT_, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, ex, stream)
   switch (rt * 10 + nt) {
     case 11: KVC_SKINNY(1, 1); break;
     case 12: KVC_SKINNY(1, 2); break;
@@ -299,14 +427,14 @@ int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int 
 
 // silu(A Wg^T) * (A Wu^T) with Wg the first N rows of W and Wu the next N
 int dispatch_gated(bf16_t* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N,
-                   int K, int64_t lda, int64_t ldc, hipStream_t stream) {
+                   int K, int64_t lda, int64_t ldc, const SkinnyExtras& ex, hipStream_t stream) {
   int waves = 4;
   while (waves > 1 && K / waves < 128) waves /= 2;
   const int nt = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 63) / 64 * 64;
 #define KVC_SKINNY_GATED(NT_) \
-  launch<2, NT_, bf16_t, true>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, stream)
+  launch<2, NT_, bf16_t, true>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, ex, stream)
   switch (nt) {
     case 1: KVC_SKINNY_GATED(1); break;
     case 2: KVC_SKINNY_GATED(2); break;
@@ -319,39 +447,87 @@ int dispatch_gated(bf16_t* C, const bf16_t* A, const bf16_t* W, const bf16_t* bi
 
 }  // namespace
 
+namespace {
+
+int check_operands(const char* who, const void* A, const void* W, int M, int N, int K, int64_t lda,
+                   int64_t ldc) {
+  static thread_local char msg[160];
+  if (M < 0 || M > 64 || N <= 0 || K <= 0 || lda < K || ldc < N) {
+    snprintf(msg, sizeof(msg), "%s: bad sizes (1 to 64 rows)", who);
+    return kvc_fail(msg);
+  }
+  if (K % 8 || lda % 8) {
+    snprintf(msg, sizeof(msg), "%s: K and the row stride must be multiples of 8", who);
+    return kvc_fail(msg);
+  }
+  if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15)) {
+    snprintf(msg, sizeof(msg), "%s: operands must be 16-byte aligned", who);
+    return kvc_fail(msg);
+  }
+  return 0;
+}
+
+const SkinnyExtras kNoExtras = {nullptr, 0, 1.f, 0.f, nullptr, 0, nullptr, nullptr};
+
+}  // namespace
+
 extern "C" int kvc_gemm_skinny_silu_mul_bf16(void* C, const void* A, const void* W, const void* bias,
                                              int M, int N, int K, int64_t lda, int64_t ldc,
                                              kvc_stream stream) {
-  if (M < 0 || M > 64 || N <= 0 || K <= 0 || lda < K || ldc < N)
-    return kvc_fail("kvc_gemm_skinny_silu_mul_bf16: bad sizes (1 to 64 rows)");
-  if (K % 8 || lda % 8)
-    return kvc_fail("kvc_gemm_skinny_silu_mul_bf16: K and the row stride must be multiples of 8");
-  if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15))
-    return kvc_fail("kvc_gemm_skinny_silu_mul_bf16: operands must be 16-byte aligned");
+  if (int rc = check_operands("kvc_gemm_skinny_silu_mul_bf16", A, W, M, N, K, lda, ldc)) return rc;
   if (M == 0) return 0;
   return dispatch_gated(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
                         static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N, K,
-                        lda, ldc, reinterpret_cast<hipStream_t>(stream));
+                        lda, ldc, kNoExtras, reinterpret_cast<hipStream_t>(stream));
 }
 
 extern "C" int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M,
                                     int N, int K, int64_t lda, int64_t ldc, int out_dtype,
                                     kvc_stream stream) {
-  if (M < 0 || M > 64 || N <= 0 || K <= 0 || lda < K || ldc < N)
-    return kvc_fail("kvc_gemm_skinny_bf16: bad sizes (1 to 64 rows)");
-  if (K % 8 || lda % 8)
-    return kvc_fail("kvc_gemm_skinny_bf16: K and the row stride must be multiples of 8");
-  if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15))
-    return kvc_fail("kvc_gemm_skinny_bf16: operands must be 16-byte aligned");
+  if (int rc = check_operands("kvc_gemm_skinny_bf16", A, W, M, N, K, lda, ldc)) return rc;
   if (M == 0) return 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (out_dtype == 0)
     return dispatch<float>(static_cast<float*>(C), static_cast<const bf16_t*>(A),
                            static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N,
-                           K, lda, ldc, s);
+                           K, lda, ldc, kNoExtras, s);
   if (out_dtype == 1)
     return dispatch<bf16_t>(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
                             static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N,
-                            K, lda, ldc, s);
+                            K, lda, ldc, kNoExtras, s);
   return kvc_fail("kvc_gemm_skinny_bf16: unknown output dtype code");
+}
+
+extern "C" int kvc_gemm_skinny_blocks(int N, int K, int gated) {
+  if (N <= 0 || K <= 0) return 0;
+  if (gated) return (N + 15) / 16;
+  int rt, waves;
+  pick_shape(N, K, &rt, &waves);
+  return (N + 16 * rt - 1) / (16 * rt);
+}
+
+extern "C" int kvc_gemm_skinny_fused_bf16(void* C, const void* A, const void* W, const void* bias,
+                                          int M, int N, int K, int64_t lda, int64_t ldc, int gated,
+                                          const float* in_ss, int in_parts, int in_width,
+                                          float in_eps, float* residual, int64_t ldr,
+                                          const float* gain, float* out_ss, kvc_stream stream) {
+  if (int rc = check_operands("kvc_gemm_skinny_fused_bf16", A, W, M, N, K, lda, ldc)) return rc;
+  if ((in_ss != nullptr || residual != nullptr) && M > 16)
+    return kvc_fail("kvc_gemm_skinny_fused_bf16: norms are folded in for at most 16 rows");
+  if (in_ss != nullptr && (in_parts <= 0 || in_width <= 0))
+    return kvc_fail("kvc_gemm_skinny_fused_bf16: row scaling needs its part count and width");
+  if (residual != nullptr && (gain == nullptr || out_ss == nullptr || ldr < N || gated))
+    return kvc_fail("kvc_gemm_skinny_fused_bf16: the residual form needs gain and out_ss, rows of "
+                    "at least N, and is not gated");
+  if (M == 0) return 0;
+  SkinnyExtras ex = {in_ss, in_parts, static_cast<float>(in_width), in_eps,
+                     residual, ldr, gain, out_ss};
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (gated)
+    return dispatch_gated(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
+                          static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N, K,
+                          lda, ldc, ex, s);
+  return dispatch<bf16_t>(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
+                          static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N, K,
+                          lda, ldc, ex, s);
 }

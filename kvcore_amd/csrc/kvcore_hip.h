@@ -128,6 +128,22 @@ int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias
 int kvc_gemm_skinny_silu_mul_bf16(void* C, const void* A, const void* W, const void* bias, int M,
                                   int N, int K, int64_t lda, int64_t ldc, kvc_stream stream);
 
+// The same products with the RMS norm of the rows folded in, for steps of at most 16 tokens,
+// so that no separate norm kernel runs between them:
+//  - in_ss [M, in_parts] (or null): A holds rows with the norm's gain applied but not yet
+//    normalised; row m's sums are multiplied by rsqrt(sum_p in_ss[m, p] / in_width + in_eps)
+//    before bias (and activation);
+//  - residual [M, ldr] float32 (or null; not with gated): residual += product (+ bias); C
+//    receives bfloat16(residual * gain[n]) and out_ss [M, blocks] the new residual's sums of
+//    squares per block of columns, blocks = kvc_gemm_skinny_blocks(N, K, 0): the in_ss of the
+//    product that consumes C.
+// gated = 1 is kvc_gemm_skinny_silu_mul_bf16's product (N = the gate's rows).
+int kvc_gemm_skinny_blocks(int N, int K, int gated);
+int kvc_gemm_skinny_fused_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
+                               int K, int64_t lda, int64_t ldc, int gated, const float* in_ss,
+                               int in_parts, int in_width, float in_eps, float* residual,
+                               int64_t ldr, const float* gain, float* out_ss, kvc_stream stream);
+
 // table[triples[3i], triples[3i+1]] = triples[3i+2] for i < n.
 int kvc_table_update(int32_t* table, int table_stride, int table_rows, const int32_t* triples,
                      int n, kvc_stream stream);

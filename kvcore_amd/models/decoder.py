@@ -172,8 +172,9 @@ class DecoderModel:
             pe.prepare(ctx)
             pe.embed(residual, ctx)
         delta = None
-        for call in self.calls:
-            delta = self.blocks[call.layer_index].forward(delta, residual, ctx, call)
+        for i, call in enumerate(self.calls):
+            nxt = self.blocks[self.calls[i + 1].layer_index] if i + 1 < len(self.calls) else None
+            delta = self.blocks[call.layer_index].forward(delta, residual, ctx, call, next_block=nxt)
         hidden = ctx.buf("final_hidden", H)
         self.final_norm.forward_fused(hidden, residual, delta)
         return hidden

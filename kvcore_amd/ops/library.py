@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_float, c_int, c_int64, c_void_p
+from dataclasses import dataclass
 
 import torch
 
@@ -49,6 +50,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
         "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, P],
         "kvc_gemm_skinny_silu_mul_bf16": [P, P, P, P, I, I, I, L, L, P],
+        "kvc_gemm_skinny_blocks": [I, I, I],
+        "kvc_gemm_skinny_fused_bf16": [P, P, P, P, I, I, I, L, L, I, P, I, I, F, P, L, P, P, P],
         "kvc_table_update": [P, I, I, P, I, P],
         "kvc_argmax": [P, P, I, I, L, P, P, I, P],
         "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P],
@@ -384,16 +387,115 @@ def gemm_skinny_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor,
            "kvc_gemm_skinny_bf16")
 
 
+@dataclass
+class ScaledRows:
+    """Activation rows ``[T, H]`` that carry an RMS norm still to be finished: ``data`` holds
+    ``residual * gain`` in bfloat16, ``ss_parts`` ``[T, parts]`` float32 partial sums of the
+    residual's squares.  ``linear`` and ``linear_silu_mul`` take it in place of ``x`` and
+    multiply row ``t``'s sums by ``rsqrt(sum(ss_parts[t]) / width + eps)``, which equals
+    the product of the normalised row.  Made by ``linear`` into a :class:`ResidualSink`."""
+
+    data: torch.Tensor
+    ss_parts: torch.Tensor
+    width: int
+    eps: float
+
+    @property
+    def shape(self) -> torch.Size:
+        return self.data.shape
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.data.dtype
+
+
+@dataclass
+class ResidualSink:
+    """Where a product's result may go instead of a plain tensor: added into the float32
+    ``residual`` rows, with ``out`` receiving ``bfloat16(residual * gain)`` and ``ss_parts``
+    (room for ``[T, parts]`` float32) the new rows' partial sums of squares: the next norm,
+    done but for the scale factor that the consuming product applies."""
+
+    residual: torch.Tensor
+    gain: torch.Tensor
+    eps: float
+    out: torch.Tensor
+    ss_parts: torch.Tensor
+
+
+def rows_fusable(num_rows: int, dtype: torch.dtype) -> bool:
+    """Whether a step of ``num_rows`` tokens may hand its norms to the products around them."""
+    return dtype == torch.bfloat16 and 0 < num_rows <= SKINNY_PREFERRED_ROWS
+
+
+def skinny_blocks(N: int, K: int, gated: bool = False) -> int:
+    """How many blocks of columns the weight-streaming kernel cuts ``N`` outputs into."""
+    return int(load().kvc_gemm_skinny_blocks(N, K, int(gated)))
+
+
+def _fused_skinny(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: torch.Tensor,
+                  bias: torch.Tensor | None, gated: bool) -> ScaledRows | None:
+    """The weight-streaming product with a norm on either side folded in (see the C header)."""
+    data = x.data if isinstance(x, ScaledRows) else x
+    M, K = data.shape
+    N = w.shape[0] // 2 if gated else w.shape[0]
+    if data.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != K:
+        raise KernelError("fused product: operands must be bfloat16 of matching width")
+    if not _skinny_operands_ok(data, w):
+        raise KernelError("fused product: at most 64 rows, K a multiple of 8, 16-byte aligned operands")
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != w.shape[0]):
+        raise KernelError("fused product: bias must be bfloat16, one per weight row")
+    in_ss = in_parts = in_width = 0
+    in_eps = 0.0
+    if isinstance(x, ScaledRows):
+        in_parts = x.ss_parts.shape[1]
+        if x.ss_parts.shape[0] < M or x.ss_parts.dtype != torch.float32 or not x.ss_parts.is_contiguous():
+            raise KernelError("fused product: ss_parts must be contiguous float32 [>= T, parts]")
+        in_ss, in_width, in_eps = x.ss_parts.data_ptr(), x.width, x.eps
+    result = None
+    if isinstance(out, ResidualSink):
+        parts = skinny_blocks(N, K)
+        if out.residual.shape != (M, N) or out.residual.dtype != torch.float32 or out.residual.stride(1) != 1:
+            raise KernelError("fused product: the residual must be float32 [T, N]")
+        if out.gain.shape != (N,) or out.gain.dtype != torch.float32:
+            raise KernelError("fused product: the gain must be float32 [N]")
+        if out.out.shape != (M, N) or out.out.dtype != torch.bfloat16 or out.out.stride(1) != 1:
+            raise KernelError("fused product: the sink's rows must be bfloat16 [T, N]")
+        if out.ss_parts.numel() < M * parts or out.ss_parts.dtype != torch.float32 \
+                or not out.ss_parts.is_contiguous():
+            raise KernelError("fused product: the sink's ss_parts is too small")
+        ss_view = out.ss_parts.view(-1)[: M * parts].view(M, parts)
+        c_ptr, ldc = out.out.data_ptr(), out.out.stride(0)
+        residual, ldr, gain, out_ss = (out.residual.data_ptr(), out.residual.stride(0),
+                                       out.gain.data_ptr(), ss_view.data_ptr())
+        result = ScaledRows(out.out, ss_view, N, out.eps)
+    else:
+        if out.shape != (M, N) or out.dtype != torch.bfloat16 or out.stride(1) != 1:
+            raise KernelError("fused product: out must be bfloat16 [T, N]")
+        c_ptr, ldc = out.data_ptr(), out.stride(0)
+        residual = gain = out_ss = None
+        ldr = 0
+    if M:
+        _check(load().kvc_gemm_skinny_fused_bf16(
+            c_ptr, data.data_ptr(), _dev(w, "w"), None if bias is None else _dev(bias, "bias"), M, N, K,
+            data.stride(0), ldc, int(gated), in_ss or None, in_parts, in_width, float(in_eps),
+            residual, ldr, gain, out_ss, _stream()), "kvc_gemm_skinny_fused_bf16")
+    return result
+
+
 def _skinny_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return (x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def linear_silu_mul(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None,
-                    scratch) -> None:
+def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Tensor,
+                    bias: torch.Tensor | None, scratch) -> None:
     """``out = silu(x @ wg.T) * (x @ wu.T)`` with ``wg`` the first half of ``w``'s rows and
     ``wu`` the second (biases likewise).  Few rows of bfloat16 run as one weight-streaming
     kernel; otherwise ``scratch()`` gives the ``[M, 2I]`` buffer for the two-kernel form."""
+    if isinstance(x, ScaledRows):
+        _fused_skinny(out, x, w, bias, gated=True)
+        return
     M, K = x.shape
     I = w.shape[0] // 2
     if w.shape != (2 * I, K) or out.shape != (M, I):
@@ -414,11 +516,16 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: t
     silu_mul(out, gate_up)
 
 
-def linear(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -> None:
+def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: torch.Tensor,
+           bias: torch.Tensor | None = None) -> ScaledRows | None:
     """``out = x @ w.T (+ bias)``.  float32 runs the library's own true-float32 kernel.
     bfloat16 with at most 64 rows runs the weight-streaming matrix-core kernel (float32
     ``out`` allowed); more rows run the vendor matrix product through torch.  All sum in
-    float32."""
+    float32.  With a :class:`ScaledRows` for ``x`` or a :class:`ResidualSink` for ``out``
+    (few rows of bfloat16 only) the norm before or after the product is folded into it; a
+    sink returns the :class:`ScaledRows` it made."""
+    if isinstance(x, ScaledRows) or isinstance(out, ResidualSink):
+        return _fused_skinny(out, x, w, bias, gated=False)
     if x.dtype == torch.float32:
         gemm_f32(out, x, w, bias)
         return

@@ -36,6 +36,14 @@ class PagedAttention(Mixer):
     """``scale`` is a parameter (the reference fixes ``head_dim ** -0.5`` at
     llama3.py:60); ``window`` 0 attends to every earlier token."""
 
+    @property
+    def takes_scaled_rows(self) -> bool:  # x only goes into the qkv product
+        return self.hidden_size % 8 == 0
+
+    @property
+    def takes_sink(self) -> bool:  # the output product's rows are whole heads
+        return self.q_size % 8 == 0
+
     def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: float, bias: bool = False, window: int = 0,
                  position: PositionEncoding | None = None) -> None:
@@ -76,7 +84,7 @@ class PagedAttention(Mixer):
     def cache_need(self) -> CacheNeed:
         return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x: torch.Tensor, ctx, call) -> torch.Tensor:
+    def forward(self, x, ctx, call, sink=None):
         p = self.params
         qkv = ctx.buf("attn_qkv", self.q_size + 2 * self.kv_size)
         ops.linear(qkv, x, p["qkv_proj.weight"], p.get("qkv_proj.bias"))
@@ -131,6 +139,8 @@ class PagedAttention(Mixer):
                                       d=self.head_dim, scale=self.scale, window=self.window)
             else:
                 ops.paged_attention(attn, qkv, k_cache, v_cache, **common)
+        if sink is not None:
+            return ops.linear(sink, attn, p["o_proj.weight"], p.get("o_proj.bias"))
         out = ctx.buf("mixer_out", self.hidden_size)
         ops.linear(out, attn, p["o_proj.weight"], p.get("o_proj.bias"))
         return out

@@ -107,11 +107,19 @@ class Part:
 
 class Norm(Part):
     """``forward_fused`` adds ``delta`` (may be None) into the float32 ``residual`` in
-    place and writes the normalised rows into ``out`` (model dtype)."""
+    place and writes the normalised rows into ``out`` (model dtype).
+
+    ``as_gain`` returns ``(gain [H] float32, eps)`` if the norm is ``x * rsqrt(mean(x^2) +
+    eps) * gain``, so that the products around it may do its work (a product's epilogue adds
+    into the residual and keeps the sums of squares, the next product applies the scale
+    factor); None keeps the norm a step of its own."""
 
     def forward_fused(self, out: torch.Tensor, residual: torch.Tensor,
                       delta: torch.Tensor | None) -> None:
         raise NotImplementedError
+
+    def as_gain(self) -> "tuple[torch.Tensor, float] | None":
+        return None
 
 
 class PositionEncoding(Part):
@@ -139,7 +147,15 @@ class RotaryTables:
 
 class Mixer(Part):
     """Mixes information across the tokens of a request.  ``x`` is ``[T, hidden]`` in
-    the model dtype; the result has the same shape and may live in a step buffer."""
+    the model dtype; the result has the same shape and may live in a step buffer.
+
+    ``takes_scaled_rows``: ``x`` may also be an ``ops.ScaledRows`` (rows whose norm the first
+    product finishes), because the part only hands ``x`` to ``ops.linear``.  ``takes_sink``:
+    ``forward`` has a keyword ``sink`` (an ``ops.ResidualSink`` or None); given one, the last
+    product goes into it and its ``ScaledRows`` is returned instead of a tensor."""
+
+    takes_scaled_rows = False
+    takes_sink = False
 
     def cache_need(self) -> CacheNeed | None:
         return None
@@ -152,6 +168,11 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    """``takes_scaled_rows`` and ``takes_sink`` as for :class:`Mixer`."""
+
+    takes_scaled_rows = False
+    takes_sink = False
+
     def forward(self, x: torch.Tensor, ctx: "StepContext", call: "LayerCall") -> torch.Tensor:
         raise NotImplementedError
 
@@ -170,8 +191,15 @@ class Block(Part):
         """Checkpoint sub-prefix -> part."""
         raise NotImplementedError
 
+    def input_gain(self) -> "tuple[torch.Tensor, float] | None":
+        """``(gain, eps)`` of the block's first norm if the block before may hand over its
+        result as ``ops.ScaledRows`` made for that norm (see :meth:`Norm.as_gain`), else None."""
+        return None
+
     def forward(self, delta: torch.Tensor | None, residual: torch.Tensor, ctx: "StepContext",
-                call: "LayerCall") -> torch.Tensor:
+                call: "LayerCall", next_block: "Block | None" = None) -> torch.Tensor:
+        """``next_block`` is the block that runs after this one (None after the last); the
+        result may be ``ops.ScaledRows`` only if ``next_block.input_gain()`` allowed it."""
         raise NotImplementedError
 
 

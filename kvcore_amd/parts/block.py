@@ -10,6 +10,8 @@ from __future__ import annotations
 
 import torch
 
+from kvcore_amd.ops import library as ops
+
 from .base import Block, FeedForward, Mixer, Norm, Part, register_block
 
 
@@ -36,12 +38,41 @@ class PreNormBlock(Block):
             self.ffn_name: self.ffn,
         }
 
-    def forward(self, delta: torch.Tensor | None, residual: torch.Tensor, ctx, call) -> torch.Tensor:
-        x = ctx.buf("block_x", residual.shape[1])
-        self.norms[self.NORM_NAMES[0]].forward_fused(x, residual, delta)
-        a = self.mixer.forward(x, ctx, call)
-        self.norms[self.NORM_NAMES[1]].forward_fused(x, residual, a)
-        return self.ffn.forward(x, ctx, call)
+    def input_gain(self):
+        gain = self.norms[self.NORM_NAMES[0]].as_gain()
+        return gain if gain is not None and self.mixer.takes_scaled_rows else None
+
+    @staticmethod
+    def _sink(ctx, residual: torch.Tensor, gain, name: str) -> ops.ResidualSink:
+        H = residual.shape[1]
+        rows = ctx.buf(name, H)
+        parts = ctx.buffers.get(name + "_ss", ops.SKINNY_PREFERRED_ROWS, -(-H // 16), torch.float32)
+        return ops.ResidualSink(residual, gain[0], gain[1], rows, parts)
+
+    def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
+        # With few rows of bfloat16 the norms fold into the products around them: the product
+        # before a norm adds into the residual and keeps the sums of squares, the product after
+        # it applies the scale factor.  Otherwise every norm is a kernel of its own.
+        fold = ops.rows_fusable(ctx.num_tokens, ctx.dtype) and residual.shape[1] % 8 == 0
+        if isinstance(delta, ops.ScaledRows):
+            x = delta  # the block before made the first norm's rows
+        else:
+            x = ctx.buf("block_x", residual.shape[1])
+            self.norms[self.NORM_NAMES[0]].forward_fused(x, residual, delta)
+
+        post = self.norms[self.NORM_NAMES[1]]
+        gain = post.as_gain() if fold and self.mixer.takes_sink and self.ffn.takes_scaled_rows else None
+        if gain is not None:
+            x2 = self.mixer.forward(x, ctx, call, sink=self._sink(ctx, residual, gain, "block_x2"))
+        else:
+            a = self.mixer.forward(x, ctx, call)
+            x2 = ctx.buf("block_x2", residual.shape[1])
+            post.forward_fused(x2, residual, a)
+
+        gain = next_block.input_gain() if fold and next_block is not None and self.ffn.takes_sink else None
+        if gain is not None:
+            return self.ffn.forward(x2, ctx, call, sink=self._sink(ctx, residual, gain, "block_x"))
+        return self.ffn.forward(x2, ctx, call)
 
 
 register_block("prenorm", PreNormBlock)

@@ -14,6 +14,14 @@ from .base import FeedForward, ParamSource, ParamSpec, register_feed_forward
 
 
 class SwiGLU(FeedForward):
+    @property
+    def takes_scaled_rows(self) -> bool:  # x only goes into the gate-up product
+        return self.hidden_size % 8 == 0
+
+    @property
+    def takes_sink(self) -> bool:
+        return self.intermediate_size % 8 == 0
+
     def __init__(self, *, hidden_size: int, intermediate_size: int, bias: bool = False) -> None:
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
@@ -34,12 +42,14 @@ class SwiGLU(FeedForward):
             specs.append(ParamSpec("down_proj.bias", (H,), init="zeros"))
         return specs
 
-    def forward(self, x: torch.Tensor, ctx, call) -> torch.Tensor:
+    def forward(self, x, ctx, call, sink=None):
         p = self.params
         act = ctx.buf("ffn_act", self.intermediate_size)
         # few rows: the product and the activation are one kernel and gate_up is never stored
         ops.linear_silu_mul(act, x, p["gate_up_proj.weight"], p.get("gate_up_proj.bias"),
                             lambda: ctx.buf("ffn_gate_up", 2 * self.intermediate_size))
+        if sink is not None:
+            return ops.linear(sink, act, p["down_proj.weight"], p.get("down_proj.bias"))
         out = ctx.buf("ffn_out", self.hidden_size)
         ops.linear(out, act, p["down_proj.weight"], p.get("down_proj.bias"))
         return out

@@ -26,6 +26,9 @@ class RMSNorm(Norm):
                       delta: torch.Tensor | None) -> None:
         ops.add_rmsnorm(out, residual, delta, self.params["weight"], self.eps)
 
+    def as_gain(self) -> tuple[torch.Tensor, float]:
+        return self.params["weight"], self.eps
+
     def forward_rows(self, out: torch.Tensor, x: torch.Tensor) -> None:
         """Normalise rows of ``x`` (model dtype) without a residual."""
         ops.rmsnorm(out, x, self.params["weight"], self.eps)

@@ -732,3 +732,55 @@ def test_sample_follows_the_probabilities_and_top_k_top_p_vectors(ops):
     p_logits = torch.tensor([[10.0, 9.0, 0.0, -1.0]], device=DEV).repeat(200, 1)
     got = set(sample_rows(ops, p_logits, [1.0] * 200, [0] * 200, [0.8] * 200, [1] * 200, list(range(200))))
     assert got == {0, 1}
+
+
+@pytest.mark.parametrize("M,H,I", [(1, 64, 48), (8, 4096, 1024), (16, 136, 200), (5, 4104, 88)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_norms_folded_into_the_products_around_them(ops, M, H, I, with_bias):
+    """residual += x1 W1^T; x2 = rmsnorm(residual) * gain; y = silu(x2 Wg^T) * (x2 Wu^T), once
+    with the norm as a kernel of its own and once folded into the two products."""
+    eps = 1e-5
+    x1 = rnd(M, I, dtype=torch.bfloat16, seed=1)
+    w1 = rnd(H, I, dtype=torch.bfloat16, seed=2, scale=0.1)
+    b1 = rnd(H, dtype=torch.bfloat16, seed=3) if with_bias else None
+    w2 = rnd(2 * I, H, dtype=torch.bfloat16, seed=4, scale=0.05)
+    b2 = rnd(2 * I, dtype=torch.bfloat16, seed=5) if with_bias else None
+    w3 = rnd(I, H, dtype=torch.bfloat16, seed=6, scale=0.05)
+    gain = (1 + 0.1 * rnd(H, dtype=torch.float32, seed=7))
+    residual0 = 3 * rnd(M, H, dtype=torch.float32, seed=8)
+
+    # folded
+    res = residual0.clone()
+    rows = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    parts = torch.full((16, -(-H // 16)), float("nan"), device=DEV)
+    scaled = ops.linear(ops.ResidualSink(res, gain, eps, rows, parts), x1, w1, b1)
+    assert isinstance(scaled, ops.ScaledRows) and scaled.ss_parts.shape == (M, ops.skinny_blocks(H, I))
+    y = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear_silu_mul(y, scaled, w2, b2, None)
+    z = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear(z, scaled, w3)
+
+    # the formula in float64
+    r = residual0.double() + x1.double() @ w1.double().T + (b1.double() if with_bias else 0.0)
+    assert torch.allclose(res.double(), r, atol=1e-4, rtol=1e-5)
+    assert torch.allclose(scaled.ss_parts.double().sum(1), (r * r).sum(1), rtol=1e-5)
+    x2 = plain.rms_norm(r, gain.double(), eps)
+    want_y = plain.silu_and_mul(x2 @ w2.double().T + (b2.double() if with_bias else 0.0))
+    want_z = x2 @ w3.double().T
+    def close(got, want):  # bfloat16 activations: each element within 2% of the row's scale
+        err = (got.double() - want).abs()
+        return bool((err <= 2e-2 * want.abs().amax(dim=1, keepdim=True) + 1e-3).all()) and \
+            float(err.norm() / want.norm()) < 1e-2
+
+    assert close(y, want_y)
+    assert close(z, want_z)
+
+    # and the unfolded kernels agree with the folded ones to bfloat16 rounding
+    res2 = residual0.clone()
+    delta = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
+    ops.linear(delta, x1, w1, b1)
+    x2b = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
+    ops.add_rmsnorm(x2b, res2, delta, gain, eps)
+    z2 = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
+    ops.linear(z2, x2b, w3)
+    assert close(z, z2.double())
