@@ -94,7 +94,14 @@ def _check(code: int, name: str) -> None:
         raise KernelError(f"{name} failed ({code}): {msg}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """The current stream's handle (asked of torch at every launch: a stream context or a
+    graph capture may have changed it)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
