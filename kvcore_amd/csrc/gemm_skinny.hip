@@ -125,6 +125,25 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) row_scale[nt] = 1.f;
 
+  // the residual rows this block will add into, asked for now by the wave that adds at the
+  // end: they were written by the kernel before and come from far
+  f32x4_t res_pre[RT][NT];
+  bool res_vec[RT][NT];
+  if constexpr ((FOLD & 2) != 0) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int n_first = n0 + rt * 16 + 4 * quad;
+        const int tok = nt * 16 + col;
+        const float* rp = ex.residual + static_cast<int64_t>(tok < M ? tok : 0) * ex.ldr + n_first;
+        res_vec[rt][nt] = wave == 0 && tok < M && N - n_first >= 4 &&
+                          (reinterpret_cast<uintptr_t>(rp) & 15) == 0;
+        res_pre[rt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if (res_vec[rt][nt]) res_pre[rt][nt] = *reinterpret_cast<const f32x4_t*>(rp);
+      }
+  }
+
   // Whole steps of 64 along K first, software-pipelined: the loads of the next STAGES - 1
   // steps are in flight while a step is multiplied (a lane reads 2 x 16 bytes = a row reads
   // 128 contiguous bytes a step).  Then whole 32-wide steps, then one guarded step for a
@@ -303,12 +322,12 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
           if (tok >= M || n_left <= 0) continue;
           float* rp = ex.residual + static_cast<int64_t>(tok) * ex.ldr + n_first;
           bf16_t* cp = reinterpret_cast<bf16_t*>(C) + static_cast<int64_t>(tok) * ldc + n_first;
-          if (n_left >= 4 && ((reinterpret_cast<uintptr_t>(rp) | reinterpret_cast<uintptr_t>(ex.gain + n_first)) & 15) == 0 &&
+          if (res_vec[rt][nt] && (reinterpret_cast<uintptr_t>(ex.gain + n_first) & 15) == 0 &&
               (reinterpret_cast<uintptr_t>(cp) & 7) == 0) {
             f32x4_t b = f32x4_t{0.f, 0.f, 0.f, 0.f};
             if (bias != nullptr)
               for (int i = 0; i < 4; ++i) b[i] = to_float(bias[n_first + i]);
-            const f32x4_t r = *reinterpret_cast<const f32x4_t*>(rp) + (acc[rt][nt] * row_scale[nt] + b);
+            const f32x4_t r = res_pre[rt][nt] + (acc[rt][nt] * row_scale[nt] + b);
             *reinterpret_cast<f32x4_t*>(rp) = r;
             store4<bf16_t>(cp, r * *reinterpret_cast<const f32x4_t*>(ex.gain + n_first), 4);
             ss[nt] += (r[0] * r[0] + r[1] * r[1]) + (r[2] * r[2] + r[3] * r[3]);
