@@ -161,6 +161,9 @@ class ModelRunner:
         self._graph_buckets = _decode_buckets(min(max_num_seqs, max_num_tokens))
         self._graphs: dict[tuple[int, int], tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self._graph_warm: set[tuple[int, int]] = set()
+        # one memory pool for what library calls allocate while a graph is captured (the
+        # vendor matrix product's workspace): graphs never run at the same time, so they share
+        self._graph_pool = None
         self.graph_replays = 0
 
     def _drop_graphs(self) -> None:
@@ -169,6 +172,7 @@ class ModelRunner:
             torch.cuda.synchronize(self.device)
             self._graphs.clear()
             self._graph_warm.clear()
+            self._graph_pool = None  # the pool goes with its last graph
 
     # -------------------------------------------------------------------- bookkeeping
     def forget(self, slot: int) -> None:
@@ -407,7 +411,9 @@ class ModelRunner:
         gc_was_enabled = gc.isenabled()
         gc.disable()
         try:
-            with torch.cuda.graph(graph):
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
                 logits = run()
         finally:
             if gc_was_enabled:
