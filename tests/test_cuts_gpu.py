@@ -272,3 +272,43 @@ def test_decoding_across_a_length_class(models, dtype):
         assert session.runner.graph_replays >= 90  # two classes, each: one step eager, one captured
         # the longer class is there (the shorter one's graph goes when a step buffer grows)
         assert -(-(1100 + 192) // 64) * 64 in {key[1] for key in session.runner._graphs}
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
+def test_graphs_of_wide_decode_steps_replay_right_every_time(models, dtype):
+    """Twenty requests decode together, so that the captured step holds the vendor matrix
+    product (more than 16 rows) beside our kernels.  Every replay is compared with the plain
+    implementation, and a step of another shape runs launch by launch between replays."""
+    folder, cfg, weights, page = models["D"]
+    n_req = 20
+    seqs = {f"w{i}": random_tokens(9 + 3 * i + 12, cfg["vocab_size"], seed=700 + i) for i in range(n_req)}
+    total = sum(-(-len(t) // 64) * 64 for t in seqs.values())
+    session = session_for(folder, dtype, page, max_tokens=total, max_num_seqs=24)
+    expect = {rid: oracle("D", cfg, weights, t) for rid, t in seqs.items()}
+    steps, k = [], 0
+    # prompts, four requests a step
+    ids = list(seqs)
+    for i in range(0, n_req, 4):
+        steps.append({"step": k, "end": [], "entries": [
+            {"id": r, "tokens": seqs[r][:len(seqs[r]) - 12], "want": [len(seqs[r]) - 13]} for r in ids[i:i + 4]]})
+        k += 1
+    # twelve decode steps of all twenty; after the sixth, a step of two tokens for one request
+    # (run launch by launch) stands between the replays
+    fed = {r: len(seqs[r]) - 12 for r in ids}
+    for j in range(11):
+        entries = []
+        for r in ids:
+            if j == 6 and r == ids[0]:
+                continue
+            entries.append({"id": r, "tokens": [seqs[r][fed[r]]], "want": [0]})
+            fed[r] += 1
+        steps.append({"step": k, "end": [], "entries": entries}); k += 1
+        if j == 6:
+            r = ids[0]
+            steps.append({"step": k, "end": [], "entries": [
+                {"id": r, "tokens": seqs[r][fed[r]:fed[r] + 2], "want": [0, 1]}]}); k += 1
+            fed[r] += 2
+    got = collect(session, steps)
+    compare(got, expect, dtype)
+    if session.runner.use_hip_graphs:
+        assert session.runner.graph_replays >= 8

@@ -784,3 +784,33 @@ def test_norms_folded_into_the_products_around_them(ops, M, H, I, with_bias):
     z2 = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
     ops.linear(z2, x2b, w3)
     assert close(z, z2.double())
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 4096, 14336), (24, 6144, 4096), (48, 4096, 4096), (33, 1024, 8192)])
+def test_library_product_inside_a_graph_replays_right(ops, M, N, K):
+    """Steps of more than 16 rows use the vendor matrix product, also inside captured graphs
+    (some of its kernels split K over blocks and need a workspace).  Every replay, with other
+    work between, must give the bits of the call outside a graph."""
+    w = rnd(N, K, dtype=torch.bfloat16, seed=1, scale=0.05)
+    x = rnd(M, K, dtype=torch.bfloat16, seed=2)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(out, x, w)
+    want = out.clone()
+    assert torch.allclose(want.double(), x.double() @ w.double().T, atol=0.3, rtol=3e-2)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        ops.linear(out, x, w)  # warm-up on the capturing stream
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            ops.linear(out, x, w)
+    torch.cuda.current_stream().wait_stream(stream)
+    other = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    for i in range(4):
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {i}"
+        ops.linear(other, rnd(M, K, dtype=torch.bfloat16, seed=10 + i), w)  # eager work between
+        torch.cuda.synchronize()
