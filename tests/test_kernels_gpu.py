@@ -814,3 +814,63 @@ def test_library_product_inside_a_graph_replays_right(ops, M, N, K):
         assert torch.equal(out, want), f"replay {i}"
         ops.linear(other, rnd(M, K, dtype=torch.bfloat16, seed=10 + i), w)  # eager work between
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("nsplit", [1, 7, 32])
+def test_decode_attention_long_context(ops, nsplit):
+    """Twenty thousand keys: many blocks a wave, a wide block table, many parts."""
+    dtype = torch.bfloat16
+    nh, nkv, d, page = 8, 2, 128, 16
+    seq_lens = [20000, 4099, 1]
+    R = len(seq_lens)
+    kc, vc, table, dense = paged_setup(seq_lens, nkv, d, page, dtype, seed=3)
+    q = rnd(R, nh * d, dtype=dtype, seed=4)
+    positions = torch.tensor([n - 1 for n in seq_lens], dtype=torch.int32, device=DEV)
+    token_req = torch.arange(R, dtype=torch.int32, device=DEV)
+    slots = torch.arange(1, R + 1, dtype=torch.int32, device=DEV)
+    out = torch.full((R, nh * d), float("nan"), dtype=dtype, device=DEV)
+    part_o = torch.full((R * nh * nsplit, d), float("nan"), device=DEV)
+    part_ml = torch.full((R * nh * nsplit, 2), float("nan"), device=DEV)
+    scale = d ** -0.5
+    ops.decode_attention(out, q, kc, vc, table=table, positions=positions, token_req=token_req,
+                         slots=slots, nh=nh, nkv=nkv, d=d, scale=scale, nsplit=nsplit,
+                         part_o=part_o, part_ml=part_ml)
+    got = out.double().cpu().view(R, nh, d)
+    qd = q.double().cpu().view(R, nh, d)
+    for r, n in enumerate(seq_lens):
+        k, v = dense[r][0].double(), dense[r][1].double()  # [n, nkv, d]
+        for h in range(nh):
+            p = torch.softmax((k[:, h // (nh // nkv)] @ qd[r, h]) * scale, dim=0)
+            want = p @ v[:, h // (nh // nkv)]
+            assert torch.allclose(got[r, h], want, atol=1e-2, rtol=1e-2), (n, h)
+
+
+@pytest.mark.parametrize("nh,nkv,d,whole", [(8, 2, 128, 2100), (8, 1, 64, 2100), (32, 8, 128, 4200)])
+def test_prefill_attention_long_context_and_many_tokens(ops, nh, nkv, d, whole):
+    """A portion of 700 tokens after 6,000 others, and a whole prompt of thousands of tokens:
+    hundreds of key tiles; the last case has enough tokens and kv heads that the kernel takes
+    its larger query tiles."""
+    dtype, page = torch.bfloat16, 16
+    seq_lens = [6700, whole]
+    q_lens = [700, whole]
+    kc, vc, table, dense = paged_setup(seq_lens, nkv, d, page, dtype, seed=5)
+    T = sum(q_lens)
+    q = rnd(T, nh * d, dtype=dtype, seed=6)
+    positions = torch.tensor(list(range(6000, 6700)) + list(range(whole)), dtype=torch.int32, device=DEV)
+    q_start = torch.tensor([0, 700, 700 + whole], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([1, 2], dtype=torch.int32, device=DEV)
+    out = torch.full((T, nh * d), float("nan"), dtype=dtype, device=DEV)
+    scale = d ** -0.5
+    ops.prefill_attention(out, q, kc, vc, table=table, positions=positions, q_start=q_start,
+                          slots=slots, num_reqs=2, nh=nh, nkv=nkv, d=d, scale=scale)
+    assert not torch.isnan(out).any()
+    got = out.double().cpu().view(T, nh, d)
+    qd = q.double().cpu().view(T, nh, d)
+    g = nh // nkv
+    for t in [0, 1, 15, 16, 333, 699, 700, 701, 731, 732, 1500, T - 1]:  # rows at tile edges and inside
+        r = 0 if t < 700 else 1
+        pos = int(positions[t])
+        k, v = dense[r][0].double()[: pos + 1], dense[r][1].double()[: pos + 1]
+        for h in (0, nh - 1):
+            p = torch.softmax((k[:, h // g] @ qd[t, h]) * scale, dim=0)
+            assert torch.allclose(got[t, h], p @ v[:, h // g], atol=1e-2, rtol=1e-2), (t, h)
