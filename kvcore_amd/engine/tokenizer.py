@@ -42,6 +42,9 @@ class TokenizerManager:
         eos = getattr(self.tokenizer, "eos_token_id", None)
         if isinstance(eos, int):
             out.add(eos)
-        for e in getattr(self.tokenizer, "eos_token_ids", None) or []:
+        more = getattr(self.tokenizer, "eos_token_ids", None)
+        if isinstance(more, int):
+            more = [more]
+        for e in more or []:
             out.add(int(e))
         return out

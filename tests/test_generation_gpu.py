@@ -165,3 +165,34 @@ def test_command_line(folders, tmp_path):
     line = next(l for l in text.splitlines() if l.startswith("token_ids="))
     got = [int(x) for x in line.split("=", 1)[1].strip("()").split(",") if x.strip()]
     assert got == plain.greedy_generate(cfg, weights, first_prompt, 5)
+
+
+def test_chat_messages_in_and_text_out(folders, tmp_path):
+    """With a tokenizer in the model folder a request may carry chat messages: the chat
+    template makes the prompt, the tokenizer's end-of-sequence id stops generation, and the
+    output comes back as text (reference: kvcore/entry/llm_engine.py:38-48, 97-107)."""
+    import shutil
+
+    from kvcore_amd import SamplingParams
+    from kvcore_amd.engine.llm_engine import GenerationRequest
+    from tests.test_tokenizer import make_tokenizer_folder
+
+    src, cfg, weights, page = folders["A"]
+    folder = tmp_path / "with_tokenizer"
+    shutil.copytree(src, folder)
+    words = make_tokenizer_folder(folder)
+    engine = make_engine(folder, "float32", page)
+    assert words.index("<eos>") in engine.engine_core.stop_token_ids
+    messages = ({"role": "user", "content": "hello world how are you"},)
+    out = engine.generate([GenerationRequest("chat", SamplingParams(max_tokens=12, temperature=0.0),
+                                             messages=messages)])[0]
+    prompt = [words.index(w) for w in ["<|user|>", "hello", "world", "how", "are", "you", "<|assistant|>"]]
+    check_tokens(cfg, weights, prompt, list(out.output_token_ids), temperature=0.0, seed=0, tol=1e-4)
+    assert isinstance(out.output_text, str)
+    if out.finish_reason == "stop":
+        assert out.output_token_ids[-1] == words.index("<eos>")
+    else:
+        assert out.finish_reason == "length" and len(out.output_token_ids) == 12
+    # a request without a tokenizer-made prompt needs token ids
+    with pytest.raises(ValueError):
+        engine.generate([GenerationRequest("bad", SamplingParams(max_tokens=2))])
