@@ -1,8 +1,10 @@
 // Sampling over float32 logits: one block of 1024 threads per row.
 //
 // Greedy is the argmax (lowest index among equals).  Otherwise the row is divided by
-// its temperature; top-k and top-p become a value threshold found by 32 halvings over
-// the order-preserving integer image of float32 (no sort); the token is
+// its temperature; top-k and top-p become a value threshold found digit by digit (four
+// digits of eight bits, a histogram in LDS each: counts for top-k, probability mass in
+// fixed point for top-p) over the order-preserving integer image of float32, without a
+// sort and with sums that do not depend on the order of addition; the token is
 // argmax_v(z_v - log(e_v)) with e_v = -log(u_v) exponential noise, which is the same
 // draw as argmax_v(softmax(z)_v / e_v).  u_v comes from 32-bit integer mixing of
 // (seed, output index, v), so a row's draw depends on nothing else in the batch.
@@ -43,6 +45,28 @@ __device__ __forceinline__ float uniform_noise(uint32_t key, uint32_t v) {
 __device__ __forceinline__ uint32_t order_key(float f) {
   const uint32_t b = __float_as_uint(f);
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+// f(v, row[v]) for every v < V, this thread's share: four values a load where the row is
+// aligned, several loads in flight
+template <typename F>
+__device__ __forceinline__ void for_each_logit(const float* __restrict__ row, int V, F f) {
+  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const int V4 = V >> 2;
+    const float4* row4 = reinterpret_cast<const float4*>(row);
+#pragma unroll 4
+    for (int i = threadIdx.x; i < V4; i += kThreads) {
+      const float4 x = row4[i];
+      f(4 * i, x.x);
+      f(4 * i + 1, x.y);
+      f(4 * i + 2, x.z);
+      f(4 * i + 3, x.w);
+    }
+    for (int v = 4 * V4 + threadIdx.x; v < V; v += kThreads) f(v, row[v]);
+  } else {
+#pragma unroll 4
+    for (int v = threadIdx.x; v < V; v += kThreads) f(v, row[v]);
+  }
 }
 
 struct Best {
@@ -91,7 +115,7 @@ __global__ __launch_bounds__(kThreads) void argmax_kernel(int32_t* __restrict__ 
   __shared__ Best scratch[kThreads / kWave];
   const float* row = logits + static_cast<int64_t>(blockIdx.x) * row_stride;
   Best mine{-INFINITY, -1};
-  for (int v = threadIdx.x; v < V; v += kThreads) mine = better(mine, Best{row[v], v});
+  for_each_logit(row, V, [&](int v, float x) { mine = better(mine, Best{x, v}); });
   const Best total = block_best(mine, scratch);
   if (threadIdx.x == 0) out[blockIdx.x] = total.idx < 0 ? 0 : total.idx;
 }
@@ -146,7 +170,7 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(
 
   if (temp < kGreedyEps) {
     Best mine{-INFINITY, -1};
-    for (int v = threadIdx.x; v < V; v += kThreads) mine = better(mine, Best{row[v], v});
+    for_each_logit(row, V, [&](int v, float x) { mine = better(mine, Best{x, v}); });
     const Best total = block_best(mine, best_scratch);
     if (threadIdx.x == 0) out[s] = total.idx < 0 ? 0 : total.idx;
     return;
@@ -157,57 +181,104 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(
   const float p_keep = top_p[s];
 
   // threshold key: entries with order_key(z) >= keep_key stay
+  __shared__ unsigned long long hist[256];
+  __shared__ uint32_t chosen_prefix;
+  __shared__ unsigned long long chosen_sum;
   uint32_t keep_key = 0u;
   if (k < V) {
-    // the k-th largest value: the largest key with at least k entries at or above it
-    uint32_t lo = 0u;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = lo | (1u << bit);
-      float cnt = 0.f;
-      for (int v = threadIdx.x; v < V; v += kThreads)
-        cnt += (order_key(row[v] * inv_t) >= cand) ? 1.f : 0.f;
-      const float total = block_sum(cnt, f_scratch);
-      if (total >= static_cast<float>(k)) lo = cand;
+    // the k-th largest key, digit by digit from the top: among the entries that share the
+    // digits found so far, the highest digit with at least `need` entries at or above it
+    uint32_t prefix = 0u;
+    unsigned long long need = static_cast<unsigned long long>(k);
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      for (int b = threadIdx.x; b < 256; b += kThreads) hist[b] = 0ull;
+      __syncthreads();
+      const uint32_t high_mask = (shift == 24) ? 0u : (0xFFFFFFFFu << (shift + 8));
+      for_each_logit(row, V, [&](int, float x) {
+        const uint32_t key = order_key(x * inv_t);
+        if ((key & high_mask) == (prefix & high_mask)) atomicAdd(&hist[(key >> shift) & 255u], 1ull);
+      });
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        unsigned long long above = 0ull;
+        int d = 255;
+        for (; d > 0; --d) {
+          if (above + hist[d] >= need) break;
+          above += hist[d];
+        }
+        chosen_prefix = prefix | (static_cast<uint32_t>(d) << shift);
+        chosen_sum = need - above;  // still to find among the entries of this digit
+      }
+      __syncthreads();
+      prefix = chosen_prefix;
+      need = chosen_sum;
     }
-    keep_key = lo;
+    keep_key = prefix;
   }
   if (p_keep < 1.0f) {
     float zmax = -INFINITY;
-    for (int v = threadIdx.x; v < V; v += kThreads) zmax = fmaxf(zmax, row[v] * inv_t);
+    for_each_logit(row, V, [&](int, float x) { zmax = fmaxf(zmax, x * inv_t); });
     zmax = block_max(zmax, f_scratch);
     const uint32_t max_key = order_key(zmax);
-    float den = 0.f;
-    for (int v = threadIdx.x; v < V; v += kThreads) {
-      const float z = row[v] * inv_t;
-      if (order_key(z) >= keep_key) den += expf(z - zmax);
-    }
-    den = block_sum(den, f_scratch);
-    const float limit = (1.0f - p_keep) * den;
-    // the largest key whose strictly-smaller kept entries weigh at most `limit`
-    uint32_t lo = 0u;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = lo | (1u << bit);
-      float mass = 0.f;
-      for (int v = threadIdx.x; v < V; v += kThreads) {
-        const float z = row[v] * inv_t;
+    // probability mass in fixed point (2^-40 of the largest entry's), so that sums are exact
+    // integers whatever the order of addition
+    constexpr float kFix = 1099511627776.0f;  // 2^40
+    unsigned long long den = 0ull;
+    for_each_logit(row, V, [&](int, float x) {
+      const float z = x * inv_t;
+      if (order_key(z) >= keep_key) den += static_cast<unsigned long long>(expf(z - zmax) * kFix);
+    });
+    for (int b = threadIdx.x; b < 256; b += kThreads) hist[b] = 0ull;
+    __syncthreads();
+    atomicAdd(&hist[0], den);
+    __syncthreads();
+    den = hist[0];
+    const unsigned long long limit =
+        static_cast<unsigned long long>((1.0 - static_cast<double>(p_keep)) * static_cast<double>(den));
+    // the largest key whose strictly-smaller kept entries weigh at most `limit`, digit by digit
+    uint32_t prefix = 0u;
+    unsigned long long below = 0ull;  // mass of the kept entries whose key is under `prefix`
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      __syncthreads();
+      for (int b = threadIdx.x; b < 256; b += kThreads) hist[b] = 0ull;
+      __syncthreads();
+      const uint32_t high_mask = (shift == 24) ? 0u : (0xFFFFFFFFu << (shift + 8));
+      for_each_logit(row, V, [&](int, float x) {
+        const float z = x * inv_t;
         const uint32_t key = order_key(z);
-        if (key >= keep_key && key < cand) mass += expf(z - zmax);
+        if (key >= keep_key && (key & high_mask) == (prefix & high_mask)) {
+          const unsigned long long m = static_cast<unsigned long long>(expf(z - zmax) * kFix);
+          if (m) atomicAdd(&hist[(key >> shift) & 255u], m);
+        }
+      });
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        unsigned long long run = below;
+        int d = 0;
+        for (; d < 255; ++d) {
+          if (run + hist[d] > limit) break;
+          run += hist[d];
+        }
+        chosen_prefix = prefix | (static_cast<uint32_t>(d) << shift);
+        chosen_sum = run;
       }
-      mass = block_sum(mass, f_scratch);
-      if (mass <= limit) lo = cand;
+      __syncthreads();
+      prefix = chosen_prefix;
+      below = chosen_sum;
     }
+    uint32_t lo = prefix;
     if (lo > max_key) lo = max_key;  // the largest entry is never dropped
     if (lo > keep_key) keep_key = lo;
   }
 
   const uint32_t key = noise_key(seed_lo[s], seed_hi[s], index[s]);
   Best mine{-INFINITY, -1};
-  for (int v = threadIdx.x; v < V; v += kThreads) {
-    const float z = row[v] * inv_t;
-    if (order_key(z) < keep_key) continue;
+  for_each_logit(row, V, [&](int v, float x) {
+    const float z = x * inv_t;
+    if (order_key(z) < keep_key) return;
     const float e = -logf(uniform_noise(key, static_cast<uint32_t>(v)));
     mine = better(mine, Best{z - logf(e), v});
-  }
+  });
   const Best total = block_best(mine, best_scratch);
   if (threadIdx.x == 0) out[s] = total.idx < 0 ? 0 : total.idx;
 }
