@@ -61,6 +61,9 @@ def parse_args():
     p.add_argument("--mixed", action="store_true",
                    help="instead of the decode runs: 64 requests with prompts of 16..2048 tokens, "
                         "portions of 512, 128 new tokens each, timed as a whole")
+    p.add_argument("--long-prompt", type=int, default=0, metavar="N",
+                   help="time to the first token of one N-token prompt, in portions of 2,048 "
+                        "tokens; prints its own line")
     p.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     p.add_argument("--only-prefill", action="store_true",
                    help="run only the 2,048-token prefill (for profiling); prints its own line")
@@ -117,8 +120,11 @@ def main() -> int:
 
     max_seqs = 64
     pages_per_seq = -(-(PREFILL_TOKENS + NEW_TOKENS + prompt_len) // PAGE_SIZE)
+    if args.long_prompt:
+        max_seqs, pages_per_seq = 2, -(-(args.long_prompt + 16) // PAGE_SIZE)
     engine = EngineCore(KVCoreConfig(
-        model_config=ModelConfig(model=".", dtype=args.dtype, max_model_len=CONTEXT_LEN),
+        model_config=ModelConfig(model=".", dtype=args.dtype,
+                                 max_model_len=max(CONTEXT_LEN, args.long_prompt + 16)),
         load_config=LoadConfig(load_format="random", seed=0),
         cache_config=CacheConfig(block_size=PAGE_SIZE, num_gpu_blocks=max_seqs * pages_per_seq + 1),
         scheduler_config=SchedulerConfig(max_num_seqs=max_seqs, max_num_scheduled_tokens=PREFILL_TOKENS,
@@ -176,6 +182,21 @@ def main() -> int:
             drain()
         return sorted(times[1:])[1]  # median of the three after the warm-up run
 
+    if args.long_prompt:
+        times = []
+        for i in range(3):
+            new_request(args.long_prompt, 1)
+            torch.cuda.synchronize()
+            t_start = time.perf_counter()
+            drain()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t_start)
+        sec = min(times[1:])
+        print(json.dumps({"workload": f"first token of a {args.long_prompt}-token prompt in portions of "
+                                      f"{PREFILL_TOKENS}", "model": model_name, "dtype": args.dtype,
+                          "ms": round(sec * 1e3, 2), "tokens_per_s": round(args.long_prompt / sec, 1),
+                          "frac": round(prefill_flops(cfg, args.long_prompt) / sec / PEAK_FLOPS[args.dtype], 4)}))
+        return 0
     if args.mixed:
         lens = [rng.randrange(16, 2049) for _ in range(64)]
         engine.scheduler.config = SchedulerConfig(

@@ -29,6 +29,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include "attention_combine.h"
 #include "device_utils.h"
 #include "kvcore_hip.h"
 
@@ -407,7 +408,7 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
 // out[t, head, :] = sum_s w_s * part_o[s] / sum_s w_s * l_s with w_s = exp2(m_s - max m).
 // Every wave works the weights out for itself (lane s holds split s), so nothing waits on
 // another wave; the partial outputs are asked for before the weights are known.
-constexpr int kMaxSplits = 64;
+constexpr int kMaxSplits = kMaxAttentionSplits;
 __global__ void decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                                       const float* __restrict__ part_ml, int D, int nsplit) {
   const int64_t th = blockIdx.x;  // token * nh + head
@@ -469,6 +470,16 @@ int launch_decode(DecodeArgs& args, int T, hipStream_t stream) {
 }
 
 }  // namespace
+
+int kvc::launch_attention_combine(bf16_t* out, const float* part_o, const float* part_ml, int64_t rows,
+                                  int d, int nsplit, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (rows > 0x7fffffff || nsplit < 1 || nsplit > kMaxAttentionSplits)
+    return kvc_fail("attention combine: bad sizes");
+  hipLaunchKernelGGL(decode_combine_kernel, dim3(static_cast<unsigned>(rows)), dim3((d + 63) / 64 * 64), 0,
+                     stream, out, part_o, part_ml, d, nsplit);
+  return kvc_check_launch("attention combine");
+}
 
 extern "C" int kvc_decode_attention_supported(int nh, int nkv, int d, int page_size, int dtype) {
   if (dtype != 1) return 0;

@@ -21,6 +21,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include "attention_combine.h"
 #include "device_utils.h"
 #include "kvcore_hip.h"
 
@@ -57,7 +58,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ table, int table_stride, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int num_reqs, int nh,
-    int nkv, int page_size, int num_pages, float scale_log2e, int window) {
+    int nkv, int page_size, int num_pages, float scale_log2e, int window,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int NJ = D / 16;
   constexpr int NC = D / 32;
   constexpr int KROW = D + 8;  // padded K row in LDS (elements)
@@ -405,21 +407,42 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     }
   };
 
-  fetch_tile(kb_first);
-  store_tile(0);
-  __syncthreads();
-  int buf = 0;
-  for (int kb0 = kb_first; kb0 < kb_end; kb0 += kKeyBlocks, buf ^= 1) {
-    const bool more = kb0 + kKeyBlocks < kb_end;
-    if (more) fetch_tile(kb0 + kKeyBlocks);  // in flight while this tile is used
-    if (kb0 * 16 <= wave_pos_hi) work_tile(kb0, buf);  // scalar: else nothing here is visible to this wave
-    if (more) store_tile(buf ^ 1);
-    __syncthreads();  // the next tile is whole, and this one has been consumed
+  // With gridDim.z > 1 the key tiles of the rows are dealt to that many blocks in
+  // consecutive runs; each leaves its unnormalised sums for the combining kernel.
+  const int tiles_all = (kb_end - kb_first + kKeyBlocks - 1) / kKeyBlocks;
+  const int tiles_mine = (tiles_all + static_cast<int>(gridDim.z) - 1) / static_cast<int>(gridDim.z);
+  const int kb_mine = kb_first + static_cast<int>(blockIdx.z) * tiles_mine * kKeyBlocks;
+  const int kb_mine_end = (kb_mine + tiles_mine * kKeyBlocks < kb_end) ? kb_mine + tiles_mine * kKeyBlocks : kb_end;
+  if (kb_mine < kb_mine_end) {  // the same for the whole block
+    fetch_tile(kb_mine);
+    store_tile(0);
+    __syncthreads();
+    int buf = 0;
+    for (int kb0 = kb_mine; kb0 < kb_mine_end; kb0 += kKeyBlocks, buf ^= 1) {
+      const bool more = kb0 + kKeyBlocks < kb_mine_end;
+      if (more) fetch_tile(kb0 + kKeyBlocks);  // in flight while this tile is used
+      if (kb0 * 16 <= wave_pos_hi) work_tile(kb0, buf);  // scalar: else nothing here is visible to this wave
+      if (more) store_tile(buf ^ 1);
+      __syncthreads();  // the next tile is whole, and this one has been consumed
+    }
   }
 
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     if (!live[ct]) continue;
+    if (gridDim.z > 1) {
+      // sums relative to m, and m in the exponent's units, as the combining kernel expects
+      const int64_t slot =
+          (static_cast<int64_t>(my_tok[ct]) * nh + my_head[ct]) * gridDim.z + blockIdx.z;
+      float* po = part_o + slot * D + 4 * quad;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) *reinterpret_cast<f32x4_t*>(po + 16 * j) = o_acc[ct][j];
+      if (quad == 0) {
+        part_ml[2 * slot] = (m[ct] == -INFINITY) ? -INFINITY : m[ct] * scale_log2e;
+        part_ml[2 * slot + 1] = l[ct];
+      }
+      continue;
+    }
     const float inv = (l[ct] > 0.f) ? 1.f / l[ct] : 0.f;
     bf16_t* op = out + (static_cast<int64_t>(my_tok[ct]) * nh + my_head[ct]) * D + 4 * quad;
 #pragma unroll
@@ -437,7 +460,7 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
                       const bf16_t* v_cache, const int32_t* table, int table_stride,
                       const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                       int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
-                      hipStream_t stream) {
+                      float* part_o, float* part_ml, int nsplit, hipStream_t stream) {
   const int g = nh / nkv;
   const int bq = (64 * CT) / g;
   // every request may end in a ragged tile and have an odd number of tiles
@@ -447,9 +470,11 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
       reinterpret_cast<const void*>(&prefill_attention_kernel<D, CT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
   if (attr != hipSuccess) return kvc_fail("kvc_prefill_attention: the kernel's LDS size was refused");
-  hipLaunchKernelGGL((prefill_attention_kernel<D, CT>), dim3(max_pairs, nkv), dim3(kWaves * 64),
+  hipLaunchKernelGGL((prefill_attention_kernel<D, CT>), dim3(max_pairs, nkv, nsplit), dim3(kWaves * 64),
                      lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
-                     q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window);
+                     q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, part_o,
+                     part_ml);
+  if (nsplit > 1) return launch_attention_combine(out, part_o, part_ml, static_cast<int64_t>(T) * nh, D, nsplit, stream);
   return kvc_check_launch("kvc_prefill_attention");
 }
 
@@ -458,19 +483,20 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
                    const bf16_t* v_cache, const int32_t* table, int table_stride,
                    const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                    int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
-                   hipStream_t stream) {
+                   float* part_o, float* part_ml, int nsplit, hipStream_t stream) {
   const int g = nh / nkv;
   // Tiles of 128 query rows stage each key tile for twice the rows, tiles of 64 make twice
-  // the blocks: the larger ones once their pairs alone give every compute unit two blocks.
+  // the blocks: the larger ones once their blocks alone give every compute unit two, and
+  // whenever the keys are split (the caller splits until there are blocks enough).
   const int bq2 = 128 / g > 0 ? 128 / g : 1;
   const int64_t pairs2 = static_cast<int64_t>(((T + bq2 - 1) / bq2 + 1) / 2) * nkv;
-  if (pairs2 >= 512 || g > 64)
+  if (pairs2 >= 512 || nsplit > 1 || g > 64)
     return launch_prefill_ct<D, 2>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                                    q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window,
-                                   stream);
+                                   part_o, part_ml, nsplit, stream);
   return launch_prefill_ct<D, 1>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                                  q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window,
-                                 stream);
+                                 part_o, part_ml, nsplit, stream);
 }
 
 }  // namespace
@@ -488,7 +514,7 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
                                      const int32_t* positions, const int32_t* q_start,
                                      const int32_t* slots, int T, int R, int nh, int nkv, int d,
                                      int page_size, int num_pages, float scale, int window,
-                                     kvc_stream stream) {
+                                     void* part_o, void* part_ml, int nsplit, kvc_stream stream) {
   if (!kvc_prefill_attention_supported(nh, nkv, d, page_size, 1))
     return kvc_fail("kvc_prefill_attention: unsupported shape (bfloat16, head size 64 or 128, at "
                     "most 64 query heads per kv head, page size a multiple of 16)");
@@ -496,7 +522,13 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
     return kvc_fail("kvc_prefill_attention: bad sizes");
   if (!(scale > 0.f)) return kvc_fail("kvc_prefill_attention: the scale must be positive");
   if (q_stride % 8) return kvc_fail("kvc_prefill_attention: q rows must be 16-byte aligned");
+  if (nsplit < 1 || nsplit > kMaxAttentionSplits)
+    return kvc_fail("kvc_prefill_attention: between 1 and 64 splits");
+  if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr))
+    return kvc_fail("kvc_prefill_attention: splits need a workspace");
   if (T == 0) return 0;
+  float* po = static_cast<float*>(part_o);
+  float* pml = static_cast<float*>(part_ml);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bf16_t* qq = static_cast<const bf16_t*>(q);
   const bf16_t* kc = static_cast<const bf16_t*>(k_cache);
@@ -504,8 +536,8 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
   if (d == 64)
     return launch_prefill<64>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                               positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                              window, s);
+                              window, po, pml, nsplit, s);
   return launch_prefill<128>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                              positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                             window, s);
+                             window, po, pml, nsplit, s);
 }

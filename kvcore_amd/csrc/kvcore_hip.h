@@ -102,13 +102,17 @@ int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* qkv
 // The same attention for bfloat16 portions of prompts on the matrix cores: a block per
 // (tile of a request's tokens, kv head), keys staged through LDS.  q_start [R+1] bounds
 // each request's tokens in the flattened batch; slots [R] names its block-table row;
-// positions must rise by one along a request's tokens.
+// positions must rise by one along a request's tokens.  With nsplit > 1 the keys of every
+// tile are dealt to that many blocks (for few query rows against many keys) and a second
+// kernel joins their results; part_o [T*nh*nsplit, d] and part_ml [T*nh*nsplit, 2] float32
+// are its workspace.
 int kvc_prefill_attention_supported(int nh, int nkv, int d, int page_size, int dtype);
 int kvc_prefill_attention(void* out, const void* q, int64_t q_stride, const void* k_cache,
                           const void* v_cache, const int32_t* table, int table_stride,
                           const int32_t* positions, const int32_t* q_start, const int32_t* slots,
                           int T, int R, int nh, int nkv, int d, int page_size, int num_pages,
-                          float scale, int window, kvc_stream stream);
+                          float scale, int window, void* part_o, void* part_ml, int nsplit,
+                          kvc_stream stream);
 
 // C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) in float32 with float32 products and sums;
 // each element is one running sum over k = 0..K-1, whatever M is.

@@ -45,7 +45,7 @@ def _declare(lib: ctypes.CDLL) -> None:
                                  F, I, I, P],
         "kvc_decode_attention_waves": [I, I, I],
         "kvc_decode_attention_supported": [I, I, I, I, I],
-        "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
+        "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, P, I, P],
         "kvc_prefill_attention_supported": [I, I, I, I, I],
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
         "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, P],
@@ -326,8 +326,11 @@ def prefill_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype
 def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       *, table: torch.Tensor, positions: torch.Tensor, q_start: torch.Tensor,
                       slots: torch.Tensor, num_reqs: int, nh: int, nkv: int, d: int, scale: float,
-                      window: int = 0) -> None:
-    """bfloat16 attention of portions of prompts on the matrix cores (see the C header)."""
+                      window: int = 0, nsplit: int = 1, part_o: torch.Tensor | None = None,
+                      part_ml: torch.Tensor | None = None) -> None:
+    """bfloat16 attention of portions of prompts on the matrix cores (see the C header).
+    ``nsplit > 1`` deals every tile's keys to that many blocks; ``part_o`` (float32,
+    ``T*nh*nsplit*d`` values) and ``part_ml`` (``T*nh*nsplit*2``) are then the workspace."""
     T = out.shape[0]
     if out.shape != (T, nh * d) or not out.is_contiguous() or out.dtype != torch.bfloat16:
         raise KernelError("prefill_attention: out must be contiguous bfloat16 [T, nh*d]")
@@ -338,11 +341,17 @@ def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         raise KernelError("prefill_attention: cache dtype differs from the queries'")
     if positions.numel() < T or q_start.numel() < num_reqs + 1 or slots.numel() < num_reqs:
         raise KernelError("prefill_attention: index arrays too short")
+    po = pml = None
+    if nsplit > 1:
+        if part_o is None or part_ml is None or part_o.numel() < T * nh * nsplit * d or \
+                part_ml.numel() < T * nh * nsplit * 2:
+            raise KernelError("prefill_attention: the workspace for splits is missing or too small")
+        po, pml = _dev(part_o, "part_o", torch.float32), _dev(part_ml, "part_ml", torch.float32)
     _check(load().kvc_prefill_attention(
         out.data_ptr(), q.data_ptr(), q.stride(0), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _dev(table, "table", torch.int32), table.shape[1], _dev(positions, "positions", torch.int32),
         _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), T, num_reqs,
-        nh, nkv, d, page_size, num_pages, float(scale), int(window), _stream()),
+        nh, nkv, d, page_size, num_pages, float(scale), int(window), po, pml, int(nsplit), _stream()),
         "kvc_prefill_attention")
 
 

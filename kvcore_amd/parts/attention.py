@@ -19,6 +19,36 @@ DECODE_TARGET_BLOCKS = 256  # one block for each compute unit
 DECODE_MAX_SPLITS = 32
 
 
+def prefill_split_rows(nkv: int, g: int) -> int:
+    """An upper bound on tokens x splits when ``prefill_splits`` gives more than one split."""
+    rows_tokens = max(128 // g, 1)
+    return 4 * PREFILL_TARGET_BLOCKS * rows_tokens // nkv + 2 * rows_tokens
+
+
+PREFILL_TARGET_BLOCKS = 512
+PREFILL_MIN_KEYS = 256      # for steps of few tokens, whose partial results are small
+PREFILL_MIN_KEYS_MOST = 1024
+PREFILL_MAX_SPLITS = 32
+
+
+def prefill_splits(T: int, nkv: int, g: int, max_query_len: int, max_seq_len: int, window: int) -> int:
+    """How many blocks share the keys of one tile of query rows in the kernel for portions
+    of prompts.  One, unless the step has too few tiles of 128 query rows to give every
+    compute unit two blocks; then as many as make up for it, while every block still has
+    keys enough to walk to be worth its partial results: a few hundred, a thousand for steps
+    of thousands of tokens (a row sees ``max_seq_len`` keys at most and, under the causal
+    mask, about half a portion fewer on average)."""
+    rows_tokens = max(128 // g, 1)
+    blocks = ((-(-T // rows_tokens)) + 1) // 2 * nkv
+    if blocks >= PREFILL_TARGET_BLOCKS:
+        return 1
+    keys = max_seq_len - min(T, max_query_len) // 2
+    if window > 0:
+        keys = min(keys, window + rows_tokens)
+    min_keys = min(max(T // 2, PREFILL_MIN_KEYS), PREFILL_MIN_KEYS_MOST)
+    return max(1, min(-(-PREFILL_TARGET_BLOCKS // blocks), keys // min_keys, PREFILL_MAX_SPLITS))
+
+
 def decode_splits(num_tokens: int, num_kv_heads: int, max_seq_len: int, waves: int,
                   window: int = 0) -> int:
     """Into how many parts each request's key range is cut for the decode kernel, beyond the
@@ -132,11 +162,24 @@ class PagedAttention(Mixer):
                               nkv=self.num_kv_heads, d=self.head_dim, write_kv=call.write_cache)
             if ctx.max_query_len > 1 and self.scale > 0 and ops.prefill_attention_supported(
                     self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
-                # portions of prompts (single tokens may ride along): tiles of query rows per block
+                # portions of prompts (single tokens may ride along): tiles of query rows per
+                # block, and several blocks per tile where few rows meet many keys
+                T = ctx.num_tokens
+                nsplit = prefill_splits(T, self.num_kv_heads, self.num_heads // self.num_kv_heads,
+                                        ctx.max_query_len, ctx.max_seq_len, self.window)
+                part_o = part_ml = None
+                if nsplit > 1:
+                    # asked for at their largest at once: a buffer that grows drops the graphs
+                    most = prefill_split_rows(self.num_kv_heads, self.num_heads // self.num_kv_heads) * self.num_heads
+                    part_o = ctx.buffers.get("attn_prefill_part_o", T * self.num_heads * nsplit,
+                                             self.head_dim, torch.float32, reserve=most)
+                    part_ml = ctx.buffers.get("attn_prefill_part_ml", T * self.num_heads * nsplit, 2,
+                                              torch.float32, reserve=most)
                 ops.prefill_attention(attn, qkv, k_cache, v_cache, table=group.table,
                                       positions=ctx.positions, q_start=ctx.q_start, slots=ctx.slots,
                                       num_reqs=ctx.num_reqs, nh=self.num_heads, nkv=self.num_kv_heads,
-                                      d=self.head_dim, scale=self.scale, window=self.window)
+                                      d=self.head_dim, scale=self.scale, window=self.window,
+                                      nsplit=nsplit, part_o=part_o, part_ml=part_ml)
             else:
                 ops.paged_attention(attn, qkv, k_cache, v_cache, **common)
         if sink is not None:

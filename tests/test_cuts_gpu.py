@@ -204,6 +204,36 @@ def test_mixed_batches_with_page_reuse(models, name, dtype):
     assert session.manager.num_free_pages()[0] == session.num_pages - 1
 
 
+def test_mixed_batches_with_the_keys_of_a_tile_dealt_to_several_blocks(models, monkeypatch):
+    """Portions of prompts that meet many keys have each tile's keys dealt to several blocks,
+    joined by a second kernel.  The tiny models' contexts are short, so the number of keys a
+    block should at least have is lowered until the mixed trace runs that way."""
+    from kvcore_amd.ops import library as ops
+    from kvcore_amd.parts import attention
+
+    monkeypatch.setattr(attention, "PREFILL_MIN_KEYS", 48)
+    calls = []
+    real = ops.prefill_attention
+
+    def spy(*args, **kw):
+        calls.append(kw.get("nsplit", 1))
+        return real(*args, **kw)
+
+    monkeypatch.setattr(ops, "prefill_attention", spy)
+    name = "D"  # the tiny model whose head size the kernel for portions of prompts serves
+    folder, cfg, weights, page = models[name]
+    base = PROMPT_LENS[name]
+    lens = base + [base[-1] + 17, base[0] + 1]
+    token_lists = {f"q{i}": random_tokens(n + EXTRA, cfg["vocab_size"], seed=450 + i) for i, n in enumerate(lens)}
+    rounded = sorted((-(-len(t) // 64) * 64 for t in token_lists.values()), reverse=True)
+    session = session_for(folder, torch.bfloat16, page, max_tokens=sum(rounded[:4]))
+    got, starts = {}, {}
+    for rec in mixed_trace(token_lists, seed=6):
+        got.update(collect_one(session, rec, starts))
+    assert max(calls) > 1 and min(calls) == 1, "the trace should run with and without splits"
+    compare(got, {rid: oracle(name, cfg, weights, t) for rid, t in token_lists.items()}, torch.bfloat16)
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
 def test_logits_do_not_depend_on_which_pages_are_used(models, dtype):
     """The mixed trace again with the free pages handed out in a shuffled order: the same

@@ -557,9 +557,11 @@ def test_decode_attention_far_key_and_window(ops, nsplit):
 
 @pytest.mark.parametrize("nh,nkv,d,page", [(8, 2, 64, 16), (32, 8, 128, 16), (6, 2, 128, 32), (5, 1, 64, 48),
                                            (4, 4, 128, 16), (16, 1, 64, 16)])
-def test_prefill_attention_on_the_matrix_cores(ops, nh, nkv, d, page):
+@pytest.mark.parametrize("nsplit", [1, 3])
+def test_prefill_attention_on_the_matrix_cores(ops, nh, nkv, d, page, nsplit):
     """Portions of prompts with and without earlier context, beside single tokens, against
-    the plain attention; lengths chosen at tile, block and page edges."""
+    the plain attention; lengths chosen at tile, block and page edges.  With the keys of a
+    tile dealt to three blocks, the short requests leave some of the three without keys."""
     dtype = torch.bfloat16
     assert ops.prefill_attention_supported(nh, nkv, d, page, dtype)
     seq_lens = [200, 1, 33, 130, 64, 97, 700]
@@ -576,8 +578,11 @@ def test_prefill_attention_on_the_matrix_cores(ops, nh, nkv, d, page):
     slots = torch.arange(1, len(seq_lens) + 1, dtype=torch.int32, device=DEV)
     out = torch.full((T, nh * d), float("nan"), dtype=dtype, device=DEV)
     scale = d ** -0.5
+    part_o = torch.full((T * nh * nsplit, d), float("nan"), device=DEV)
+    part_ml = torch.full((T * nh * nsplit, 2), float("nan"), device=DEV)
     ops.prefill_attention(out, q, kc, vc, table=table, positions=positions, q_start=q_start_t,
-                          slots=slots, num_reqs=len(seq_lens), nh=nh, nkv=nkv, d=d, scale=scale)
+                          slots=slots, num_reqs=len(seq_lens), nh=nh, nkv=nkv, d=d, scale=scale,
+                          nsplit=nsplit, part_o=part_o, part_ml=part_ml)
     got = out.double().cpu().view(T, nh, d)
     qd = q.double().cpu().view(T, nh, d)
     for r, (n, ql) in enumerate(zip(seq_lens, q_lens)):
@@ -588,13 +593,15 @@ def test_prefill_attention_on_the_matrix_cores(ops, nh, nkv, d, page):
         assert torch.allclose(got[q_start[r]:q_start[r + 1]], want, atol=1e-2, rtol=1e-2), f"request {r}"
 
 
-def test_prefill_attention_far_key_and_window(ops):
+@pytest.mark.parametrize("nsplit", [1, 4])
+def test_prefill_attention_far_key_and_window(ops, nsplit):
     dtype = torch.bfloat16
     nh, nkv, d, page, n, ql = 8, 2, 64, 16, 700, 40
     positions = torch.arange(n - ql, n, dtype=torch.int32, device=DEV)
     args = dict(positions=positions, q_start=torch.tensor([0, ql], dtype=torch.int32, device=DEV),
                 slots=torch.ones(1, dtype=torch.int32, device=DEV), num_reqs=1, nh=nh, nkv=nkv, d=d,
-                scale=d ** -0.5)
+                scale=d ** -0.5, nsplit=nsplit, part_o=torch.empty(ql * nh * nsplit, d, device=DEV),
+                part_ml=torch.empty(ql * nh * nsplit, 2, device=DEV))
     for special in [0, 15, 16, 63, 64, 351, 659, 660, 698, 699]:
         kc, vc, table, dense = paged_setup([n], nkv, d, page, dtype, seed=special)
         q = rnd(ql, nh * d, dtype=dtype, seed=3)
@@ -845,11 +852,12 @@ def test_decode_attention_long_context(ops, nsplit):
             assert torch.allclose(got[r, h], want, atol=1e-2, rtol=1e-2), (n, h)
 
 
-@pytest.mark.parametrize("nh,nkv,d,whole", [(8, 2, 128, 2100), (8, 1, 64, 2100), (32, 8, 128, 4200)])
-def test_prefill_attention_long_context_and_many_tokens(ops, nh, nkv, d, whole):
+@pytest.mark.parametrize("nh,nkv,d,whole,nsplit", [(8, 2, 128, 2100, 1), (8, 1, 64, 2100, 1), (32, 8, 128, 4200, 1),
+                                                   (8, 2, 128, 2100, 7), (8, 1, 64, 2100, 2)])
+def test_prefill_attention_long_context_and_many_tokens(ops, nh, nkv, d, whole, nsplit):
     """A portion of 700 tokens after 6,000 others, and a whole prompt of thousands of tokens:
-    hundreds of key tiles; the last case has enough tokens and kv heads that the kernel takes
-    its larger query tiles."""
+    hundreds of key tiles; the third case has enough tokens and kv heads that the kernel takes
+    its larger query tiles, the last two deal each tile's keys to several blocks."""
     dtype, page = torch.bfloat16, 16
     seq_lens = [6700, whole]
     q_lens = [700, whole]
@@ -862,7 +870,9 @@ def test_prefill_attention_long_context_and_many_tokens(ops, nh, nkv, d, whole):
     out = torch.full((T, nh * d), float("nan"), dtype=dtype, device=DEV)
     scale = d ** -0.5
     ops.prefill_attention(out, q, kc, vc, table=table, positions=positions, q_start=q_start,
-                          slots=slots, num_reqs=2, nh=nh, nkv=nkv, d=d, scale=scale)
+                          slots=slots, num_reqs=2, nh=nh, nkv=nkv, d=d, scale=scale, nsplit=nsplit,
+                          part_o=torch.empty(T * nh * nsplit, d, device=DEV),
+                          part_ml=torch.empty(T * nh * nsplit, 2, device=DEV))
     assert not torch.isnan(out).any()
     got = out.double().cpu().view(T, nh, d)
     qd = q.double().cpu().view(T, nh, d)
