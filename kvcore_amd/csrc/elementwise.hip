@@ -181,6 +181,86 @@ static bool launch_add_rmsnorm_vec(T* out, float* residual, const T* delta, cons
   return true;
 }
 
+// The same with the pending output given as float32 partial sums [slices, rows, H] of a
+// product cut along K (+ a bias): they are added up in slice order, then into the residual.
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void add_slices_rmsnorm_vec_kernel(
+    T* __restrict__ out, float* __restrict__ residual, const float* __restrict__ partial, int slices,
+    int64_t slice_stride, const bf16_t* __restrict__ bias, const float* __restrict__ weight, float eps,
+    int H) {
+  __shared__ float scratch[16];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * H;
+  float v[NCH][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int e = (c * 256 + threadIdx.x) * 8;
+    if (e < H) {
+      float d[8];
+      load8(partial + base + e, d);
+      for (int s = 1; s < slices; ++s) {
+        float p[8];
+        load8(partial + s * slice_stride + base + e, p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d[i] += p[i];
+      }
+      if (bias != nullptr) {
+        float b[8];
+        load8(bias + e, b);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d[i] += b[i];
+      }
+      load8(residual + base + e, v[c]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[c][i] += d[i];
+      store8(residual + base + e, v[c]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += v[c][i] * v[c][i];
+    }
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = rsqrtf(total / static_cast<float>(H) + eps);
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int e = (c * 256 + threadIdx.x) * 8;
+    if (e < H) {
+      float w[8], y[8];
+      load8(weight + e, w);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = w[i] * (v[c][i] * inv);
+      store8(out + base + e, y);
+    }
+  }
+}
+
+extern "C" int kvc_add_slices_rmsnorm(void* out, float* residual, const float* partial, int slices,
+                                      const void* bias, const float* weight, float eps, int T, int H,
+                                      int dtype, kvc_stream stream) {
+  if (T < 0 || H <= 0 || slices < 1) return kvc_fail("kvc_add_slices_rmsnorm: bad sizes");
+  const auto misaligned = [](const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) != 0; };
+  if (H % 8 || H > 8 * 2048 || misaligned(out, 16) || misaligned(residual, 16) || misaligned(partial, 16) ||
+      misaligned(weight, 16) || (bias != nullptr && misaligned(bias, 16)))
+    return kvc_fail("kvc_add_slices_rmsnorm: the width must be a multiple of 8, at most 16384, and "
+                    "the operands 16-byte aligned");
+  if (dtype != 0 && dtype != 1) return kvc_fail("kvc_add_slices_rmsnorm: unknown dtype code");
+  if (T == 0) return 0;
+  const int nch = (H + 2047) / 2048;
+  const int64_t stride = static_cast<int64_t>(T) * H;
+  const bf16_t* b = static_cast<const bf16_t*>(bias);
+#define KVC_NORM_CASE(TT, NN)                                                                       \
+  hipLaunchKernelGGL((add_slices_rmsnorm_vec_kernel<TT, NN>), dim3(T), dim3(256), 0, S(stream),     \
+                     static_cast<TT*>(out), residual, partial, slices, stride, b, weight, eps, H)
+#define KVC_NORM_NCH(TT)                \
+  if (nch <= 1) KVC_NORM_CASE(TT, 1);   \
+  else if (nch <= 2) KVC_NORM_CASE(TT, 2); \
+  else if (nch <= 4) KVC_NORM_CASE(TT, 4); \
+  else KVC_NORM_CASE(TT, 8)
+  if (dtype == 0) { KVC_NORM_NCH(float); } else { KVC_NORM_NCH(bf16_t); }
+#undef KVC_NORM_NCH
+#undef KVC_NORM_CASE
+  return kvc_check_launch("kvc_add_slices_rmsnorm");
+}
+
 extern "C" int kvc_add_rmsnorm(void* out, float* residual, const void* delta, const float* weight,
                                float eps, int T, int H, int dtype, kvc_stream stream) {
   if (T < 0 || H <= 0) return kvc_fail("kvc_add_rmsnorm: bad sizes");

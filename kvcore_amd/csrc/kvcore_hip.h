@@ -25,6 +25,12 @@ int kvc_embed(float* residual, const void* table, const int32_t* ids, int T, int
 // rsqrt(mean(residual^2) + eps), rounded to dt.  residual stays float32.
 int kvc_add_rmsnorm(void* out, float* residual, const void* delta, const float* weight,
                     float eps, int T, int H, int dtype, kvc_stream stream);
+// The same with the pending output given as float32 partial sums [slices, T, H] of a product
+// cut along K (see kvc_gemm_mid_bf16, mode 2) and an optional bfloat16 bias [H]: the slices
+// are added up in their order, then into the residual.  H a multiple of 8, at most 16384.
+int kvc_add_slices_rmsnorm(void* out, float* residual, const float* partial, int slices,
+                           const void* bias, const float* weight, float eps, int T, int H, int dtype,
+                           kvc_stream stream);
 
 // out = weight * x * rsqrt(mean(x^2) + eps) on rows of dt (no residual), row strides given.
 int kvc_rmsnorm(void* out, const void* x, const float* weight, float eps, int T, int H,
@@ -118,6 +124,18 @@ int kvc_prefill_attention(void* out, const void* q, int64_t q_stride, const void
 // each element is one running sum over k = 0..K-1, whatever M is.
 int kvc_gemm_f32(float* C, const float* A, const float* W, const float* bias, int M, int N,
                  int K, int64_t lda, int64_t ldc, kvc_stream stream);
+
+// The same product for 17 to 64 rows, where the waves of a block share the rows of A through
+// LDS (K a multiple of 512).  mode 0: C = A W^T (+ bias), float32 (out_dtype 0) or bfloat16
+// (1).  mode 1: C[M, N] = silu(A Wg^T + bg) * (A Wu^T + bu) in bfloat16, W [2N, K] holding Wg
+// then Wu.  mode 2: narrow outputs are cut along K into kvc_gemm_mid_slices(N, K) slices and
+// only their float32 partial sums are stored, partial [slices, M, N] (no bias); the kernel
+// that consumes them adds them up in slice order.  mode 3: as mode 0, but cut along K like
+// mode 2 when `partial` is given, with a second kernel that sums the slices.
+int kvc_gemm_mid_slices(int N, int K);
+int kvc_gemm_mid_bf16(void* C, void* partial, const void* A, const void* W, const void* bias, int M,
+                      int N, int K, int64_t lda, int64_t ldc, int out_dtype, int mode,
+                      kvc_stream stream);
 
 // C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) for M <= 64 rows of bfloat16 on the matrix
 // cores, float32 sums, weights streamed once; C is float32 (out_dtype 0) or bfloat16 (1).

@@ -32,6 +32,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     sigs = {
         "kvc_embed": [P, P, P, I, I, I, I, P],
         "kvc_add_rmsnorm": [P, P, P, P, F, I, I, I, P],
+        "kvc_add_slices_rmsnorm": [P, P, P, I, P, P, F, I, I, I, P],
         "kvc_rmsnorm": [P, P, P, F, I, I, L, L, I, P],
         "kvc_residual_add": [P, P, I, I, I, P],
         "kvc_silu_mul": [P, P, I, I, I, P],
@@ -47,6 +48,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_decode_attention_supported": [I, I, I, I, I],
         "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, P, I, P],
         "kvc_prefill_attention_supported": [I, I, I, I, I],
+        "kvc_gemm_mid_slices": [I, I],
+        "kvc_gemm_mid_bf16": [P, P, P, P, P, I, I, I, L, L, I, I, P],
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
         "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, P],
         "kvc_gemm_skinny_silu_mul_bf16": [P, P, P, P, I, I, I, L, L, P],
@@ -436,7 +439,28 @@ class ResidualSink:
     gain: torch.Tensor
     eps: float
     out: torch.Tensor
-    ss_parts: torch.Tensor
+    ss_parts: torch.Tensor | None
+    # for steps of 17 to 64 rows: float32 room for the partial sums of a product cut along K
+    # (``mid_slices_bound(N) * T * N`` values); the sink then finishes the norm itself and
+    # ``out`` receives the normalised rows
+    slices: torch.Tensor | None = None
+
+
+@dataclass
+class NormedRows:
+    """Rows that a :class:`ResidualSink` has already added into the residual and normalised:
+    what ``linear`` returns for a sink in a step of 17 to 64 rows."""
+
+    data: torch.Tensor
+
+
+MID_ROWS = 64  # the most rows the weight-streaming kernels take
+
+
+def rows_sinkable(num_rows: int, dtype: torch.dtype) -> bool:
+    """Whether a step of ``num_rows`` tokens may send products into a :class:`ResidualSink`
+    that finishes the norm itself (more rows than ``rows_fusable`` allows, at most 64)."""
+    return dtype == torch.bfloat16 and SKINNY_PREFERRED_ROWS < num_rows <= MID_ROWS
 
 
 def rows_fusable(num_rows: int, dtype: torch.dtype) -> bool:
@@ -504,6 +528,91 @@ def _skinny_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+def mid_slices_bound(N: int) -> int:
+    """The most slices along K that ``gemm_mid`` cuts a weight with ``N`` rows into."""
+    return min(64, -(-256 // -(-N // 64)))
+
+
+def mid_slices(N: int, K: int) -> int:
+    """Slices along K that ``gemm_mid`` cuts an [N, K] weight into when it may (see mode 2)."""
+    return int(load().kvc_gemm_mid_slices(N, K))
+
+
+def _mid_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.shape[1] % 512 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and w.is_contiguous()
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_mid(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
+             *, mode: int = 0, partial: torch.Tensor | None = None) -> None:
+    """The weight-streaming product for 17 to 64 rows of bfloat16 (see the C header for the
+    modes: 0 plain, 1 ``silu(gate) * up``, 2 partial sums of slices along K only, 3 plain
+    with slices and a kernel that sums them)."""
+    M, K = x.shape
+    N = w.shape[0] // 2 if mode == 1 else w.shape[0]
+    if w.shape[1] != K or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not x.is_cuda:
+        raise KernelError("gemm_mid: operands must be bfloat16 GPU tensors with matching K")
+    if not _mid_operands_ok(x, w):
+        raise KernelError("gemm_mid: K must be a multiple of 512 and the operands aligned")
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != w.shape[0]):
+        raise KernelError("gemm_mid: bias must be bfloat16, one value per weight row")
+    out_ptr, ldc, code = None, N, 1
+    if mode != 2:
+        if out is None or out.shape != (M, N) or out.stride(1) != 1 or not out.is_cuda:
+            raise KernelError("gemm_mid: out does not fit")
+        out_ptr, ldc, code = out.data_ptr(), out.stride(0), _code(out, "out")
+    part_ptr = None
+    if partial is not None:
+        if partial.dtype != torch.float32 or partial.numel() < mid_slices(N, K) * M * N:
+            raise KernelError("gemm_mid: the buffer for partial sums is too small")
+        part_ptr = _dev(partial, "partial", torch.float32)
+    _check(load().kvc_gemm_mid_bf16(out_ptr, part_ptr, x.data_ptr(), _dev(w, "w"),
+                                    None if bias is None else _dev(bias, "bias"), M, N, K, x.stride(0),
+                                    ldc, code, mode, _stream()), "kvc_gemm_mid_bf16")
+
+
+def add_slices_rmsnorm(out: torch.Tensor, residual: torch.Tensor, partial: torch.Tensor, slices: int,
+                       bias: torch.Tensor | None, weight: torch.Tensor, eps: float) -> None:
+    """``residual += sum_s partial[s] (+ bias)``; ``out = rmsnorm(residual) * weight`` (see the
+    C header); ``partial`` holds ``[slices, T, H]`` float32."""
+    T, H = residual.shape
+    if out.shape != (T, H) or not out.is_contiguous() or not residual.is_contiguous():
+        raise KernelError("add_slices_rmsnorm: out and residual must be contiguous [T, H]")
+    if partial.dtype != torch.float32 or partial.numel() < slices * T * H:
+        raise KernelError("add_slices_rmsnorm: the partial sums do not fit")
+    _check(load().kvc_add_slices_rmsnorm(
+        _dev(out, "out"), _dev(residual, "residual", torch.float32), _dev(partial, "partial"), slices,
+        None if bias is None else _dev(bias, "bias", torch.bfloat16), _dev(weight, "weight", torch.float32),
+        float(eps), T, H, _code(out, "out"), _stream()), "kvc_add_slices_rmsnorm")
+
+
+def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None) -> NormedRows:
+    """A product of 17 to 64 rows into a sink: partial sums of slices along K, then one kernel
+    that adds them into the residual and normalises.  Shapes the weight-streaming kernel does
+    not take run the vendor product into the same workspace first."""
+    M, K = x.shape
+    N = w.shape[0]
+    if sink.slices is None or sink.slices.dtype != torch.float32:
+        raise KernelError("linear: a sink for more than 16 rows needs its float32 workspace")
+    if sink.residual.shape != (M, N) or sink.residual.dtype != torch.float32 or not sink.residual.is_contiguous():
+        raise KernelError("linear: the sink's residual must be contiguous float32 [T, N]")
+    if sink.out.shape != (M, N) or not sink.out.is_contiguous():
+        raise KernelError("linear: the sink's rows must be contiguous [T, N]")
+    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _mid_operands_ok(x, w) and N % 8 == 0:
+        slices = mid_slices(N, K)
+        if sink.slices.numel() < slices * M * N:
+            raise KernelError("linear: the sink's workspace is too small")
+        gemm_mid(None, x, w, mode=2, partial=sink.slices)
+        add_slices_rmsnorm(sink.out, sink.residual, sink.slices, slices, bias, sink.gain, sink.eps)
+    else:
+        if sink.slices.numel() * 2 < M * N:
+            raise KernelError("linear: the sink's workspace is too small")
+        tmp = sink.slices.view(-1).view(x.dtype)[: M * N].view(M, N)
+        linear(tmp, x, w, bias)
+        add_rmsnorm(sink.out, sink.residual, tmp, sink.gain, sink.eps)
+    return NormedRows(sink.out)
+
+
 def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Tensor,
                     bias: torch.Tensor | None, scratch) -> None:
     """``out = silu(x @ wg.T) * (x @ wu.T)`` with ``wg`` the first half of ``w``'s rows and
@@ -527,6 +636,12 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
             out.data_ptr(), x.data_ptr(), _dev(w, "w"), None if bias is None else _dev(bias, "bias"),
             M, I, K, x.stride(0), out.stride(0), _stream()), "kvc_gemm_skinny_silu_mul_bf16")
         return
+    if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+            and x.is_cuda and SKINNY_PREFERRED_ROWS < M <= MID_ROWS and _mid_operands_ok(x, w)
+            and out.stride(1) == 1):
+        # 17 to 64 rows: the waves of a block share the rows through LDS
+        gemm_mid(out, x, w, bias, mode=1)
+        return
     gate_up = scratch()
     linear(gate_up, x, w, bias)
     silu_mul(out, gate_up)
@@ -539,7 +654,10 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
     ``out`` allowed); more rows run the vendor matrix product through torch.  All sum in
     float32.  With a :class:`ScaledRows` for ``x`` or a :class:`ResidualSink` for ``out``
     (few rows of bfloat16 only) the norm before or after the product is folded into it; a
-    sink returns the :class:`ScaledRows` it made."""
+    sink returns the :class:`ScaledRows` it made, or, in a step of 17 to 64 rows, where it
+    finishes the norm itself, :class:`NormedRows`."""
+    if isinstance(out, ResidualSink) and not isinstance(x, ScaledRows) and x.shape[0] > SKINNY_PREFERRED_ROWS:
+        return _sink_mid(out, x, w, bias)
     if isinstance(x, ScaledRows) or isinstance(out, ResidualSink):
         return _fused_skinny(out, x, w, bias, gated=False)
     if x.dtype == torch.float32:

@@ -152,7 +152,8 @@ class Mixer(Part):
     ``takes_scaled_rows``: ``x`` may also be an ``ops.ScaledRows`` (rows whose norm the first
     product finishes), because the part only hands ``x`` to ``ops.linear``.  ``takes_sink``:
     ``forward`` has a keyword ``sink`` (an ``ops.ResidualSink`` or None); given one, the last
-    product goes into it and its ``ScaledRows`` is returned instead of a tensor."""
+    product goes into it through ``ops.linear`` and what that returns (``ops.ScaledRows`` or
+    ``ops.NormedRows``) is returned instead of a tensor."""
 
     takes_scaled_rows = False
     takes_sink = False
@@ -191,15 +192,18 @@ class Block(Part):
         """Checkpoint sub-prefix -> part."""
         raise NotImplementedError
 
-    def input_gain(self) -> "tuple[torch.Tensor, float] | None":
-        """``(gain, eps)`` of the block's first norm if the block before may hand over its
-        result as ``ops.ScaledRows`` made for that norm (see :meth:`Norm.as_gain`), else None."""
+    def input_gain(self, scaled: bool = True) -> "tuple[torch.Tensor, float] | None":
+        """``(gain, eps)`` of the block's first norm (see :meth:`Norm.as_gain`) if the block
+        before may do that norm's work, else None: with ``scaled`` it hands over
+        ``ops.ScaledRows`` that this block's mixer must finish, without it ``ops.NormedRows``
+        that are already normalised."""
         return None
 
     def forward(self, delta: torch.Tensor | None, residual: torch.Tensor, ctx: "StepContext",
                 call: "LayerCall", next_block: "Block | None" = None) -> torch.Tensor:
         """``next_block`` is the block that runs after this one (None after the last); the
-        result may be ``ops.ScaledRows`` only if ``next_block.input_gain()`` allowed it."""
+        result may be ``ops.ScaledRows`` or ``ops.NormedRows`` only if
+        ``next_block.input_gain()`` allowed it."""
         raise NotImplementedError
 
 

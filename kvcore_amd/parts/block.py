@@ -38,40 +38,58 @@ class PreNormBlock(Block):
             self.ffn_name: self.ffn,
         }
 
-    def input_gain(self):
+    def input_gain(self, scaled: bool = True):
+        """The first norm as (gain, eps) if the block before may do its work: leaving scaled
+        rows for this block's mixer to finish (``scaled``), or finishing it itself."""
         gain = self.norms[self.NORM_NAMES[0]].as_gain()
-        return gain if gain is not None and self.mixer.takes_scaled_rows else None
+        if scaled and not self.mixer.takes_scaled_rows:
+            return None
+        return gain
 
     @staticmethod
-    def _sink(ctx, residual: torch.Tensor, gain, name: str) -> ops.ResidualSink:
+    def _sink(ctx, residual: torch.Tensor, gain, name: str, fold: bool) -> ops.ResidualSink:
         H = residual.shape[1]
         rows = ctx.buf(name, H)
-        parts = ctx.buffers.get(name + "_ss", ops.SKINNY_PREFERRED_ROWS, -(-H // 16), torch.float32)
-        return ops.ResidualSink(residual, gain[0], gain[1], rows, parts)
+        if fold:
+            parts = ctx.buffers.get(name + "_ss", ops.SKINNY_PREFERRED_ROWS, -(-H // 16), torch.float32)
+            return ops.ResidualSink(residual, gain[0], gain[1], rows, parts)
+        slices = ctx.buffers.get("block_slices", ops.mid_slices_bound(H) * ops.MID_ROWS, H, torch.float32)
+        return ops.ResidualSink(residual, gain[0], gain[1], rows, None, slices)
 
     def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
         # With few rows of bfloat16 the norms fold into the products around them: the product
         # before a norm adds into the residual and keeps the sums of squares, the product after
         # it applies the scale factor.  Otherwise every norm is a kernel of its own.
+        # With a few dozen rows the product before a norm leaves partial sums of slices along
+        # K, and one kernel adds them into the residual and normalises.
         fold = ops.rows_fusable(ctx.num_tokens, ctx.dtype) and residual.shape[1] % 8 == 0
+        sums = ops.rows_sinkable(ctx.num_tokens, ctx.dtype) and residual.shape[1] % 8 == 0
         if isinstance(delta, ops.ScaledRows):
             x = delta  # the block before made the first norm's rows
+        elif isinstance(delta, ops.NormedRows):
+            x = delta.data  # the block before did the first norm
         else:
             x = ctx.buf("block_x", residual.shape[1])
             self.norms[self.NORM_NAMES[0]].forward_fused(x, residual, delta)
 
         post = self.norms[self.NORM_NAMES[1]]
-        gain = post.as_gain() if fold and self.mixer.takes_sink and self.ffn.takes_scaled_rows else None
+        gain = None
+        if self.mixer.takes_sink and ((fold and self.ffn.takes_scaled_rows) or sums):
+            gain = post.as_gain()
         if gain is not None:
-            x2 = self.mixer.forward(x, ctx, call, sink=self._sink(ctx, residual, gain, "block_x2"))
+            x2 = self.mixer.forward(x, ctx, call, sink=self._sink(ctx, residual, gain, "block_x2", fold))
+            if isinstance(x2, ops.NormedRows):
+                x2 = x2.data
         else:
             a = self.mixer.forward(x, ctx, call)
             x2 = ctx.buf("block_x2", residual.shape[1])
             post.forward_fused(x2, residual, a)
 
-        gain = next_block.input_gain() if fold and next_block is not None and self.ffn.takes_sink else None
+        gain = None
+        if next_block is not None and self.ffn.takes_sink and (fold or sums):
+            gain = next_block.input_gain(scaled=fold)
         if gain is not None:
-            return self.ffn.forward(x2, ctx, call, sink=self._sink(ctx, residual, gain, "block_x"))
+            return self.ffn.forward(x2, ctx, call, sink=self._sink(ctx, residual, gain, "block_x", fold))
         return self.ffn.forward(x2, ctx, call)
 
 

@@ -151,6 +151,122 @@ def test_gemm_skinny_bf16(ops, M, N, K, out_dtype):
     assert torch.equal(wide_out[:, :N], ref) and torch.all(wide_out[:, N:] == 0)
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 200, 512), (33, 64, 1024), (48, 1000, 1536), (64, 4104, 1024),
+                                   (5, 72, 512), (64, 16400, 512)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_mid_bf16(ops, M, N, K, out_dtype):
+    """The product for a few dozen rows, whose waves share the rows through LDS: at once, and
+    cut along K into partial sums that a second kernel adds up."""
+    a = rnd(M, K, dtype=torch.bfloat16, seed=1)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=2, scale=0.05)
+    bias = rnd(N, dtype=torch.bfloat16, seed=3)
+    want = a.double() @ w.double().T + bias.double()
+    mag = a.double().abs() @ w.double().abs().T + bias.double().abs()
+    bound = 8 * math.sqrt(K) * 2 ** -24 * mag + 1e-6
+    if out_dtype == torch.bfloat16:
+        bound = bound + want.abs() * 2 ** -8
+    slices = ops.mid_slices(N, K)
+    assert 1 <= slices <= ops.mid_slices_bound(N)
+    partial = torch.full((slices * M * N,), float("nan"), device=DEV)
+    outs = {}
+    for mode in (0, 3):
+        out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+        ops.gemm_mid(out, a, w, bias, mode=mode, partial=partial if mode == 3 else None)
+        err = (out.double() - want).abs()
+        assert (err <= bound).all(), (mode, float((err / bound).max()))
+        outs[mode] = out
+    # the partial sums alone: their sum in slice order is what mode 3 stored
+    ops.gemm_mid(None, a, w, mode=2, partial=partial)
+    total = partial[: slices * M * N].view(slices, M, N)[0].clone()
+    for s_ in range(1, slices):
+        total += partial[: slices * M * N].view(slices, M, N)[s_]
+    assert torch.equal((total + bias.float()).to(out_dtype), outs[3])
+    # fewer rows of the same batch give the same bits: the launch depends on N and K alone
+    few = min(M, 18)
+    out_few = torch.empty(few, N, dtype=out_dtype, device=DEV)
+    ops.gemm_mid(out_few, a[:few].contiguous(), w, bias, mode=0)
+    assert torch.equal(out_few, outs[0][:few])
+    # strided rows in and out
+    wide_in = torch.zeros(M, K + 8, dtype=torch.bfloat16, device=DEV)
+    wide_in[:, :K] = a
+    wide_out = torch.zeros(M, N + 3, dtype=out_dtype, device=DEV)
+    ops.gemm_mid(wide_out[:, :N], wide_in[:, :K], w, bias, mode=0)
+    assert torch.equal(wide_out[:, :N], outs[0]) and torch.all(wide_out[:, N:] == 0)
+
+
+@pytest.mark.parametrize("M,I,K", [(17, 72, 512), (40, 1000, 1024), (64, 8200, 512)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_gemm_mid_silu_mul(ops, M, I, K, with_bias):
+    x = rnd(M, K, dtype=torch.bfloat16, seed=1)
+    w = rnd(2 * I, K, dtype=torch.bfloat16, seed=2, scale=0.1)
+    bias = rnd(2 * I, dtype=torch.bfloat16, seed=3) if with_bias else None
+    out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear_silu_mul(out, x, w, bias, lambda: pytest.fail("the one-kernel form should have run"))
+    # both factors rounded to bfloat16 first, as the two-kernel form stores them (the two
+    # forms start their walks along K at different places, so not the same bits)
+    gu = torch.empty(M, 2 * I, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_mid(gu, x, w, bias, mode=0)
+    want = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
+    ops.silu_mul(want, gu)
+    assert torch.allclose(out.float(), want.float(), atol=2e-2, rtol=2e-2)
+    exact = x.double() @ w.double().T + (bias.double() if with_bias else 0)
+    formula = torch.nn.functional.silu(exact[:, :I]) * exact[:, I:]
+    assert torch.allclose(out.double(), formula, atol=3e-2, rtol=3e-2)
+
+
+def test_gemm_mid_refuses_what_it_does_not_take(ops):
+    a = rnd(20, 520, dtype=torch.bfloat16)
+    w = rnd(64, 520, dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelError, match="multiple of 512"):
+        ops.gemm_mid(torch.empty(20, 64, dtype=torch.bfloat16, device=DEV), a, w)
+    a = rnd(65, 512, dtype=torch.bfloat16)
+    w = rnd(64, 512, dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelError, match="1 to 64 rows"):
+        ops.gemm_mid(torch.empty(65, 64, dtype=torch.bfloat16, device=DEV), a, w)
+
+
+@pytest.mark.parametrize("T,H,slices,with_bias", [(17, 64, 1, False), (40, 1000, 3, True), (64, 4096, 4, False),
+                                                   (33, 16384, 2, True)])
+def test_add_slices_rmsnorm(ops, T, H, slices, with_bias):
+    residual = rnd(T, H, seed=1)
+    partial = rnd(slices, T, H, seed=2)
+    bias = rnd(H, dtype=torch.bfloat16, seed=3) if with_bias else None
+    weight = rnd(H, seed=4) + 1.0
+    eps = 1e-5
+    r0 = residual.clone()
+    out = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.add_slices_rmsnorm(out, residual, partial, slices, bias, weight, eps)
+    delta = partial[0].clone()
+    for s_ in range(1, slices):
+        delta += partial[s_]
+    if with_bias:
+        delta += bias.float()
+    assert torch.equal(residual, r0 + delta)  # slice order, then into the residual
+    r = residual.double()
+    want = r * torch.rsqrt((r * r).mean(dim=1, keepdim=True) + eps) * weight.double()
+    assert torch.allclose(out.double(), want, atol=1e-2, rtol=1e-2)
+
+
+def test_sink_for_a_few_dozen_rows_finishes_the_norm(ops):
+    """``linear`` into a sink with 17 to 64 rows: partial sums and one kernel that adds and
+    normalises; a width the weight-streaming kernel does not take goes through the vendor
+    product and gives the same rows beyond rounding."""
+    for M, N, K in ((20, 256, 1024), (64, 4096, 512), (33, 200, 520)):
+        x = rnd(M, K, dtype=torch.bfloat16, seed=1)
+        w = rnd(N, K, dtype=torch.bfloat16, seed=2, scale=0.05)
+        gain = rnd(N, seed=3) + 1.0
+        residual = rnd(M, N, seed=4)
+        r0 = residual.clone()
+        rows = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        work = torch.empty(ops.mid_slices_bound(N) * ops.MID_ROWS, N, device=DEV)
+        got = ops.linear(ops.ResidualSink(residual, gain, 1e-5, rows, None, work), x, w)
+        assert isinstance(got, ops.NormedRows) and got.data is rows
+        r = r0.double() + x.double() @ w.double().T
+        assert torch.allclose(residual.double(), r, atol=2e-2, rtol=1e-2)
+        want = r * torch.rsqrt((r * r).mean(dim=1, keepdim=True) + 1e-5) * gain.double()
+        assert torch.allclose(rows.double(), want, atol=3e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 16, 64), (5, 100, 200), (8, 2072, 512), (16, 88, 1032),
                                    (17, 176, 80), (64, 40, 256)])
 @pytest.mark.parametrize("with_bias", [False, True])
