@@ -9,6 +9,8 @@ products for bfloat16 excepted, which is where the reference uses a library too:
 
 from __future__ import annotations
 
+import os
+
 import ctypes
 from ctypes import c_float, c_int, c_int64, c_void_p
 from dataclasses import dataclass
@@ -440,7 +442,7 @@ class ResidualSink:
     eps: float
     out: torch.Tensor
     ss_parts: torch.Tensor | None
-    # for steps of 17 to 64 rows: float32 room for the partial sums of a product cut along K
+    # for steps of 9 to 64 rows: float32 room for the partial sums of a product cut along K
     # (``mid_slices_bound(N) * T * N`` values); the sink then finishes the norm itself and
     # ``out`` receives the normalised rows
     slices: torch.Tensor | None = None
@@ -449,7 +451,7 @@ class ResidualSink:
 @dataclass
 class NormedRows:
     """Rows that a :class:`ResidualSink` has already added into the residual and normalised:
-    what ``linear`` returns for a sink in a step of 17 to 64 rows."""
+    what ``linear`` returns for a sink that carries a workspace (steps of 9 to 64 rows)."""
 
     data: torch.Tensor
 
@@ -457,15 +459,22 @@ class NormedRows:
 MID_ROWS = 64  # the most rows the weight-streaming kernels take
 
 
-def rows_sinkable(num_rows: int, dtype: torch.dtype) -> bool:
-    """Whether a step of ``num_rows`` tokens may send products into a :class:`ResidualSink`
-    that finishes the norm itself (more rows than ``rows_fusable`` allows, at most 64)."""
-    return dtype == torch.bfloat16 and SKINNY_PREFERRED_ROWS < num_rows <= MID_ROWS
+FOLD_ROWS = 8  # up to here the few-row kernel with the norms folded in is the fastest (measured)
 
 
-def rows_fusable(num_rows: int, dtype: torch.dtype) -> bool:
-    """Whether a step of ``num_rows`` tokens may hand its norms to the products around them."""
-    return dtype == torch.bfloat16 and 0 < num_rows <= SKINNY_PREFERRED_ROWS
+def rows_fusable(num_rows: int, dtype: torch.dtype, width: int = 0) -> bool:
+    """Whether a step of ``num_rows`` tokens hands its norms to the products around them:
+    up to 8 rows, and up to 16 where the model's ``width`` is no multiple of 512, which the
+    kernel for more rows wants."""
+    most = FOLD_ROWS if width % 512 == 0 and width > 0 else SKINNY_PREFERRED_ROWS
+    return dtype == torch.bfloat16 and 0 < num_rows <= most
+
+
+def rows_sinkable(num_rows: int, dtype: torch.dtype, width: int = 0) -> bool:
+    """Whether a step of ``num_rows`` tokens sends the products before its norms into a
+    :class:`ResidualSink` that finishes the norm itself: more rows than ``rows_fusable``
+    allows, at most 64."""
+    return dtype == torch.bfloat16 and not rows_fusable(num_rows, dtype, width) and 0 < num_rows <= MID_ROWS
 
 
 def skinny_blocks(N: int, K: int, gated: bool = False) -> int:
@@ -545,7 +554,8 @@ def _mid_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 def gemm_mid(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
              *, mode: int = 0, partial: torch.Tensor | None = None) -> None:
-    """The weight-streaming product for 17 to 64 rows of bfloat16 (see the C header for the
+    """The weight-streaming product for up to 64 rows of bfloat16 whose waves share the rows
+    through LDS, the faster one from 9 rows on (see the C header for the
     modes: 0 plain, 1 ``silu(gate) * up``, 2 partial sums of slices along K only, 3 plain
     with slices and a kernel that sums them)."""
     M, K = x.shape
@@ -587,13 +597,13 @@ def add_slices_rmsnorm(out: torch.Tensor, residual: torch.Tensor, partial: torch
 
 
 def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None) -> NormedRows:
-    """A product of 17 to 64 rows into a sink: partial sums of slices along K, then one kernel
+    """A product of 9 to 64 rows into a sink: partial sums of slices along K, then one kernel
     that adds them into the residual and normalises.  Shapes the weight-streaming kernel does
     not take run the vendor product into the same workspace first."""
     M, K = x.shape
     N = w.shape[0]
     if sink.slices is None or sink.slices.dtype != torch.float32:
-        raise KernelError("linear: a sink for more than 16 rows needs its float32 workspace")
+        raise KernelError("linear: this sink needs its float32 workspace")
     if sink.residual.shape != (M, N) or sink.residual.dtype != torch.float32 or not sink.residual.is_contiguous():
         raise KernelError("linear: the sink's residual must be contiguous float32 [T, N]")
     if sink.out.shape != (M, N) or not sink.out.is_contiguous():
@@ -627,7 +637,7 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
         raise KernelError("linear_silu_mul: shapes do not match")
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and x.is_cuda and _skinny_operands_ok(x, w)
-            and (M <= 8 or (M <= SKINNY_PREFERRED_ROWS and K <= 8192))):
+            and (M <= FOLD_ROWS or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and not _mid_operands_ok(x, w)))):
         if M == 0:
             return
         if bias is not None and (bias.dtype != torch.bfloat16 or bias.shape != (2 * I,)):
@@ -637,9 +647,9 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
             M, I, K, x.stride(0), out.stride(0), _stream()), "kvc_gemm_skinny_silu_mul_bf16")
         return
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
-            and x.is_cuda and SKINNY_PREFERRED_ROWS < M <= MID_ROWS and _mid_operands_ok(x, w)
+            and x.is_cuda and FOLD_ROWS < M <= MID_ROWS and _mid_operands_ok(x, w)
             and out.stride(1) == 1):
-        # 17 to 64 rows: the waves of a block share the rows through LDS
+        # 9 to 64 rows: the waves of a block share the rows through LDS
         gemm_mid(out, x, w, bias, mode=1)
         return
     gate_up = scratch()
@@ -654,9 +664,11 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
     ``out`` allowed); more rows run the vendor matrix product through torch.  All sum in
     float32.  With a :class:`ScaledRows` for ``x`` or a :class:`ResidualSink` for ``out``
     (few rows of bfloat16 only) the norm before or after the product is folded into it; a
-    sink returns the :class:`ScaledRows` it made, or, in a step of 17 to 64 rows, where it
+    sink returns the :class:`ScaledRows` it made, or, in a step of 9 to 64 rows, where it
     finishes the norm itself, :class:`NormedRows`."""
-    if isinstance(out, ResidualSink) and not isinstance(x, ScaledRows) and x.shape[0] > SKINNY_PREFERRED_ROWS:
+    if isinstance(out, ResidualSink) and out.slices is not None:
+        if isinstance(x, ScaledRows):
+            raise KernelError("linear: a sink that finishes the norm itself takes plain rows")
         return _sink_mid(out, x, w, bias)
     if isinstance(x, ScaledRows) or isinstance(out, ResidualSink):
         return _fused_skinny(out, x, w, bias, gated=False)

@@ -57,13 +57,14 @@ class PreNormBlock(Block):
         return ops.ResidualSink(residual, gain[0], gain[1], rows, None, slices)
 
     def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
-        # With few rows of bfloat16 the norms fold into the products around them: the product
+        # With very few rows of bfloat16 the norms fold into the products around them: the product
         # before a norm adds into the residual and keeps the sums of squares, the product after
         # it applies the scale factor.  Otherwise every norm is a kernel of its own.
         # With a few dozen rows the product before a norm leaves partial sums of slices along
         # K, and one kernel adds them into the residual and normalises.
-        fold = ops.rows_fusable(ctx.num_tokens, ctx.dtype) and residual.shape[1] % 8 == 0
-        sums = ops.rows_sinkable(ctx.num_tokens, ctx.dtype) and residual.shape[1] % 8 == 0
+        H = residual.shape[1]
+        fold = ops.rows_fusable(ctx.num_tokens, ctx.dtype, H) and H % 8 == 0
+        sums = ops.rows_sinkable(ctx.num_tokens, ctx.dtype, H) and H % 8 == 0
         if isinstance(delta, ops.ScaledRows):
             x = delta  # the block before made the first norm's rows
         elif isinstance(delta, ops.NormedRows):

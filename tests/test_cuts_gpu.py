@@ -363,18 +363,21 @@ def test_steps_of_a_few_dozen_rows_on_a_wide_model(tmp_path, monkeypatch):
 
     monkeypatch.setattr(ops, "gemm_mid", spy)
     n_req = 40
-    seqs = {f"m{i}": random_tokens(5 + i % 7 + 10, cfg["vocab_size"], seed=800 + i) for i in range(n_req)}
+    tail = 3  # tokens that the first twelve requests decode after the others have ended
+    seqs = {f"m{i}": random_tokens(5 + i % 7 + 10 + (tail if i < 12 else 0), cfg["vocab_size"], seed=800 + i)
+            for i in range(n_req)}
     seqs["late"] = random_tokens(50, cfg["vocab_size"], seed=899)
     total = sum(-(-len(t) // 64) * 64 for t in seqs.values())
     session = session_for(folder, torch.bfloat16, WIDE_PAGE, max_tokens=total, max_num_seqs=48)
     expect = {rid: plain.llama_forward(cfg, weights, t, dtype=torch.float64) for rid, t in seqs.items()}
     ids = [r for r in seqs if r != "late"]
     steps, k = [], 0
+    first = {r: len(seqs[r]) - 10 - (tail if i < 12 else 0) for i, r in enumerate(ids)}
     for i in range(0, n_req, 8):
         steps.append({"step": k, "end": [], "entries": [
-            {"id": r, "tokens": seqs[r][:len(seqs[r]) - 10], "want": [len(seqs[r]) - 11]} for r in ids[i:i + 8]]})
+            {"id": r, "tokens": seqs[r][:first[r]], "want": [first[r] - 1]} for r in ids[i:i + 8]]})
         k += 1
-    fed = {r: len(seqs[r]) - 10 for r in ids}
+    fed = dict(first)
     late_at = 0
     for j in range(10):
         entries = [{"id": r, "tokens": [seqs[r][fed[r]]], "want": [0]} for r in ids]
@@ -384,8 +387,14 @@ def test_steps_of_a_few_dozen_rows_on_a_wide_model(tmp_path, monkeypatch):
             n = (9, 2, 13)[(3, 4, 7).index(j)]
             entries.append({"id": "late", "tokens": seqs["late"][late_at:late_at + n], "want": list(range(n))})
             late_at += n
-        steps.append({"step": k, "end": [], "entries": entries}); k += 1
+        steps.append({"step": k, "end": ids[12:] if j == 9 else [], "entries": entries}); k += 1
+    for j in range(tail):  # twelve rows: the same kernels from nine rows on
+        steps.append({"step": k, "end": [], "entries": [
+            {"id": r, "tokens": [seqs[r][fed[r]]], "want": [0]} for r in ids[:12]]}); k += 1
+        for r in ids[:12]:
+            fed[r] += 1
     got = collect(session, steps)
+    assert all(fed[r] == len(seqs[r]) for r in ids)
     assert 2 in modes and 1 in modes, "the partial-sum and the gated form should both have run"
     expect["late"] = expect["late"][:late_at]
     # this model's logits are larger than the tiny models' (0.46 against 0.2 in the root mean
