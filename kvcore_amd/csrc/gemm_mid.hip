@@ -106,8 +106,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mid_kernel(
     }
   };
   auto fetch_chunk = [&](int slot, int chunk) {
-    // beyond the slice: the last chunk again, never multiplied
-    const int k = 64 * where(chunk * kChunkSteps);
+    // a chunk beyond the slice: the last whole chunk again, never multiplied.  (The start is
+    // bent back by whole chunks, so that all 256 columns that are read lie inside the slice:
+    // rounds, and with them the rotation, are whole chunks.)
+    const int first = (chunk * kChunkSteps < n_steps) ? chunk * kChunkSteps : n_steps - kChunkSteps;
+    const int k = 64 * where(first);
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) areg[slot][i] = *reinterpret_cast<const bf16x8_t*>(a_src[i] + k);
   };
