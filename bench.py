@@ -7,6 +7,11 @@ batch 8 from 512-token prompts, context limit 8192.  One JSON line is printed:
 ``value`` is decoded tokens a second; ``prefill`` is a 2,048-token prompt in one step;
 ``roofline`` prices the decode step's mandatory reads (every weight once, the live
 requests' cache) against 8 TB/s; ``points`` holds decode at batch 1 and 64.
+
+Other workloads print a line of their own: ``--only-prefill``, ``--mixed`` (64 requests
+with prompts of 16 to 2,048 tokens in portions of 512), ``--long-prompt N`` (time to the
+first token of one N-token prompt in portions of 2,048); ``--model 1b|70b`` and ``--batch``
+change the shape.
 """
 
 from __future__ import annotations

@@ -258,7 +258,8 @@ struct MidPlan {
 // KVC_MID_WAVES / KVC_MID_RT / KVC_MID_SLICES override the choice for tuning.
 MidPlan plan_mid(int N, int K, bool gated, bool may_slice) {
   MidPlan p;
-  p.waves = 4;
+  // two waves a block where four would leave compute units without one
+  p.waves = (gated && (N + 63) / 64 < 192) ? 2 : 4;
   p.rt = gated ? 2 : (N >= 16384 ? 2 : 1);
   if (const char* e = getenv("KVC_MID_WAVES")) p.waves = atoi(e);
   if (const char* e = getenv("KVC_MID_RT")) p.rt = atoi(e);

@@ -179,11 +179,15 @@ int kvc_argmax(int32_t* out, const float* logits, int S, int V, int64_t row_stri
 // Per row s: temperature[s] < 1e-5 gives the argmax; otherwise
 // argmax_v(logits[v] / temperature - log(e_v)), e_v exponential noise keyed by
 // (seed_lo[s], seed_hi[s], index[s], v), over the entries that top_k[s] (<= 0: all) and
-// top_p[s] (>= 1: all) keep.
+// top_p[s] (>= 1: all) keep.  With a workspace of kvc_sample_workspace_words(S, V) 64-bit
+// words (0: rows too short to gain) every row is dealt to several blocks, which gives the
+// same draws; it need not be cleared.  filters: bit 0, some row has a top_k; bit 1, some row
+// has a top_p < 1 (passes that no row needs are left out; 3 is always right).
+int kvc_sample_workspace_words(int S, int V);
 int kvc_sample(int32_t* out, const float* logits, int S, int V, int64_t row_stride,
                const float* temperature, const int32_t* top_k, const float* top_p,
                const uint32_t* seed_lo, const uint32_t* seed_hi, const uint32_t* index,
-               kvc_stream stream);
+               void* workspace, int64_t workspace_words, int filters, kvc_stream stream);
 
 #ifdef __cplusplus
 }

@@ -59,7 +59,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_gemm_skinny_fused_bf16": [P, P, P, P, I, I, I, L, L, I, P, I, I, F, P, L, P, P, P],
         "kvc_table_update": [P, I, I, P, I, P],
         "kvc_argmax": [P, P, I, I, L, P, P, I, P],
-        "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P],
+        "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P, L, I, P],
+        "kvc_sample_workspace_words": [I, I],
     }
     for name, argtypes in sigs.items():
         fn = getattr(lib, name)
@@ -608,7 +609,11 @@ def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.
         raise KernelError("linear: the sink's residual must be contiguous float32 [T, N]")
     if sink.out.shape != (M, N) or not sink.out.is_contiguous():
         raise KernelError("linear: the sink's rows must be contiguous [T, N]")
-    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _mid_operands_ok(x, w) and N % 8 == 0:
+    # measured: the vendor product is as fast or faster once the output is wide and K is not
+    # long (8192 x 8192), and slower for narrow outputs and long K (8192 x 28672: 139 against
+    # 107 us at 64 rows; 4096 x 4096: 19 against 12)
+    ours = N < 8192 or K > 8192
+    if ours and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _mid_operands_ok(x, w) and N % 8 == 0:
         slices = mid_slices(N, K)
         if sink.slices.numel() < slices * M * N:
             raise KernelError("linear: the sink's workspace is too small")
@@ -723,9 +728,18 @@ def argmax(out: torch.Tensor, logits: torch.Tensor, part_val: torch.Tensor | Non
                              logits.stride(0), pv, pi, cap, _stream()), "kvc_argmax")
 
 
+def sample_workspace_words(S: int, V: int) -> int:
+    """64-bit words of workspace with which ``sample`` deals each row to several blocks
+    (0 for rows too short to gain from it)."""
+    return int(load().kvc_sample_workspace_words(S, V))
+
+
 def sample(out: torch.Tensor, logits: torch.Tensor, *, temperature: torch.Tensor,
            top_k: torch.Tensor, top_p: torch.Tensor, seed_lo: torch.Tensor, seed_hi: torch.Tensor,
-           index: torch.Tensor) -> None:
+           index: torch.Tensor, workspace: torch.Tensor | None = None, filters: int = 3) -> None:
+    """``workspace``: int64, ``sample_workspace_words(S, V)`` values or more, lets several
+    blocks work on a row (the same draws, sooner); ``filters`` says which of top-k (1) and
+    top-p (2) some row uses."""
     S, V = logits.shape
     if logits.stride(1) != 1 or logits.dtype != torch.float32 or not logits.is_cuda:
         raise KernelError("sample: expects float32 GPU logits [S, V]")
@@ -737,4 +751,6 @@ def sample(out: torch.Tensor, logits: torch.Tensor, *, temperature: torch.Tensor
                              _dev(temperature, "temperature", torch.float32),
                              _dev(top_k, "top_k", torch.int32), _dev(top_p, "top_p", torch.float32),
                              _dev(seed_lo, "seed_lo"), _dev(seed_hi, "seed_hi"), _dev(index, "index"),
+                             None if workspace is None else _dev(workspace, "workspace", torch.int64),
+                             0 if workspace is None else workspace.numel(), int(filters),
                              _stream()), "kvc_sample")

@@ -49,6 +49,7 @@ class Sampler:
         self._out_host = torch.empty(n, dtype=torch.int32, pin_memory=True)
         self._part_val: torch.Tensor | None = None  # workspace of the two-stage argmax
         self._part_idx: torch.Tensor | None = None
+        self._workspace: torch.Tensor | None = None  # lets several blocks sample one row
 
     def resolve_seed(self, params: SamplingParams) -> int:
         """The request's own seed, or one derived from the engine's seed and the order of
@@ -81,19 +82,27 @@ class Sampler:
             fview = buf.view(np.float32)
             uview = buf.view(np.uint32)
             V = logits.shape[1]
+            filters = 0
             for i, r in enumerate(rows):
                 p = r.params
                 fview[i] = p.temperature
                 buf[n + i] = 0 if p.top_k is None else min(p.top_k, V)
                 fview[2 * n + i] = p.top_p
+                if p.temperature >= GREEDY_EPS:
+                    filters |= (1 if p.top_k is not None and 0 < p.top_k < V else 0) | (2 if p.top_p < 1.0 else 0)
                 uview[3 * n + i] = r.seed & 0xFFFFFFFF
                 uview[4 * n + i] = (r.seed >> 32) & 0xFFFFFFFF
                 uview[5 * n + i] = r.index & 0xFFFFFFFF
             self._dev.copy_(self._host, non_blocking=True)
             d = self._dev
+            words = ops.sample_workspace_words(S, V)
+            if words and (self._workspace is None or self._workspace.numel() < words):
+                self._workspace = torch.empty(max(words, ops.sample_workspace_words(min(n, 64), V)),
+                                              dtype=torch.int64, device=self.device)
             ops.sample(out, logits, temperature=d[:n].view(torch.float32), top_k=d[n:2 * n],
                        top_p=d[2 * n:3 * n].view(torch.float32), seed_lo=d[3 * n:4 * n],
-                       seed_hi=d[4 * n:5 * n], index=d[5 * n:6 * n])
+                       seed_hi=d[4 * n:5 * n], index=d[5 * n:6 * n],
+                       workspace=self._workspace if words else None, filters=filters)
         self._out_host[:S].copy_(out, non_blocking=True)
         torch.cuda.current_stream().synchronize()
         return self._out_host[:S].tolist()

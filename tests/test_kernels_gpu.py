@@ -778,7 +778,7 @@ def test_table_update(ops):
 
 
 # -------------------------------------------------------------------------- sampling
-def sample_rows(ops, logits, temps, top_k, top_p, seeds, index):
+def sample_rows(ops, logits, temps, top_k, top_p, seeds, index, workspace=None, filters=3):
     S = logits.shape[0]
     out = torch.empty(S, dtype=torch.int32, device=DEV)
     t = lambda v, dt: torch.tensor(v, dtype=dt, device=DEV)  # noqa: E731
@@ -786,7 +786,8 @@ def sample_rows(ops, logits, temps, top_k, top_p, seeds, index):
     hi = [(s >> 32) & 0xFFFFFFFF for s in seeds]
     ops.sample(out, logits, temperature=t(temps, torch.float32), top_k=t(top_k, torch.int32),
                top_p=t(top_p, torch.float32), seed_lo=t(lo, torch.int64).to(torch.int32),
-               seed_hi=t(hi, torch.int64).to(torch.int32), index=t(index, torch.int32))
+               seed_hi=t(hi, torch.int64).to(torch.int32), index=t(index, torch.int32),
+               workspace=workspace, filters=filters)
     return out.cpu().tolist()
 
 
@@ -837,6 +838,46 @@ def test_sample_matches_the_plain_sampler_draw_for_draw(ops, V):
     # a row's draw does not depend on its batch-mates
     alone = sample_rows(ops, logits[5:6], temps[5:6], top_k[5:6], top_p[5:6], seeds[5:6], index[5:6])
     assert alone[0] == got[5]
+    assert ops.sample_workspace_words(S, V) == 0  # rows this short stay with one block each
+
+
+def test_sample_with_several_blocks_a_row_gives_the_same_draws(ops):
+    """Long rows, each dealt to several blocks through a workspace (left dirty on purpose):
+    the draws are those of one block a row and of the plain sampler, whatever passes the
+    caller says are needed."""
+    S, V = 12, 3 * 8192 + 77
+    logits = rnd(S, V, scale=2.5, seed=3)
+    logits[2, 8191] = logits[2, 8192] = 30.0  # equal largest values on either side of a chunk border
+    temps = [0.0, 0.8, 1.0, 1.7] * 3
+    top_k = [0, 0, 5, 400, 0, 3] * 2
+    top_p = [1.0, 1.0, 1.0, 0.9, 0.5, 0.3] * 2
+    seeds = [(999 + 131 * i) | ((i * 7) << 32) for i in range(S)]
+    index = [i * 5 for i in range(S)]
+    words = ops.sample_workspace_words(S, V)
+    assert words > 0
+    work = torch.full((words,), -1, dtype=torch.int64, device=DEV)
+    one_block = sample_rows(ops, logits, temps, top_k, top_p, seeds, index)
+    several = sample_rows(ops, logits, temps, top_k, top_p, seeds, index, workspace=work)
+    assert several == one_block
+    again = sample_rows(ops, logits, temps, top_k, top_p, seeds, index, workspace=work)  # a used workspace
+    assert again == one_block
+    for i in (0, 1, 2, 3, 4, 5, 9):
+        want = plain_sampling.sample(logits[i].cpu(), temperature=temps[i], top_k=top_k[i] or None,
+                                     top_p=top_p[i], seed=seeds[i], index=index[i])
+        assert several[i] == want, f"row {i}"
+    # rows without filters: the passes for them may be left out
+    plain_rows = [0, 1, 6, 7]
+    sub = lambda v: [v[i] for i in plain_rows]  # noqa: E731
+    assert all(top_k[i] == 0 and top_p[i] == 1.0 for i in plain_rows)
+    got = sample_rows(ops, logits[plain_rows], sub(temps), sub(top_k), sub(top_p), sub(seeds), sub(index),
+                      workspace=work, filters=0)
+    assert got == sub(one_block)
+    # only top-k, only top-p
+    for rows_, filt in (([2, 8], 1), ([4, 10], 2)):
+        sub = lambda v: [v[i] for i in rows_]  # noqa: E731
+        got = sample_rows(ops, logits[rows_], sub(temps), sub(top_k), sub(top_p), sub(seeds), sub(index),
+                          workspace=work, filters=filt)
+        assert got == sub(one_block)
 
 
 def test_sample_follows_the_probabilities_and_top_k_top_p_vectors(ops):
