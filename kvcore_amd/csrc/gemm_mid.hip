@@ -4,11 +4,11 @@
 // block share them through LDS instead of each reading its own copy from the cache.
 //
 // A block of WAVES waves owns WAVES * 16 * RT weight rows and a slice of K.  Each wave
-// walks its 16 * RT rows along the slice in steps of 64, with the weights of the next
-// seven steps on their way into registers (a lane loads 16 bytes of one row, a row reads
-// 128 contiguous bytes a step).  The rows of A of the slice pass through two LDS buffers
-// in chunks of 128 along K, fetched by all waves together a chunk ahead: one barrier a
-// chunk.  All loads are issued without a branch around them (addresses beyond the slice
+// walks its 16 * RT rows along the slice in steps of 64, with the weights of the next four
+// to eight steps on their way into registers (a lane loads 16 bytes of one row, a row reads
+// 128 contiguous bytes a step, and the four steps of a chunk are asked for together).  The
+// rows of A of the slice pass through two LDS buffers in chunks of 256 along K, fetched by
+// all waves together as far ahead as the weights: one barrier a chunk.  All loads are issued without a branch around them (addresses beyond the slice
 // are bent back into it and their values never multiplied), so that the waits can count
 // them exactly and none drains the queue.
 //
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mid_kernel(
   // of its steps are: by the time it is wanted in LDS it is the oldest load in flight and
   // waiting for it drains nothing.
 #pragma unroll
-  for (int st = 0; st < kStages - 1; ++st) {
+  for (int st = 0; st < kStages; ++st) {
     if (st % kChunkSteps == 0) fetch_chunk(st / kChunkSteps, st / kChunkSteps);
     load_w(st, st);
   }
@@ -146,17 +146,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mid_kernel(
   __syncthreads();
   // A slice is whole rounds of kStages steps (the host sees to it), so the body is one
   // straight line: a branch inside it would make the waits at the loop's head assume the
-  // worst and drain every load in flight once a round.
+  // worst and drain every load in flight once a round.  The weights of a whole chunk's steps
+  // are asked for together, when the chunk before them has been multiplied: a row's 512
+  // contiguous bytes then reach the memory close in time.
   for (int s0 = 0; s0 < n_steps; s0 += kStages) {
 #pragma unroll
     for (int j = 0; j < kStages; ++j) {
       const int step = s0 + j;
       const int cj = j / kChunkSteps;  // the chunk's number within the round
-      // this step's chunk was stored a chunk ago and its registers are free
-      if (j % kChunkSteps == 0) fetch_chunk(cj % AHEAD, step / kChunkSteps + AHEAD);
-      load_w((j + kStages - 1) % kStages, step + kStages - 1);
       mma_step(j, cj & 1, j % kChunkSteps);
       if (j % kChunkSteps == kChunkSteps - 1) {
+        // this chunk's registers are free: the chunk a round ahead, rows of A first
+        fetch_chunk(cj % AHEAD, step / kChunkSteps + AHEAD);
+#pragma unroll
+        for (int t = 0; t < kChunkSteps; ++t) load_w(cj * kChunkSteps + t, step + 1 - kChunkSteps + t + kStages);
         // the chunk after this one goes into the buffer that was read a chunk ago
         store_chunk((cj + 1) % AHEAD, (cj + 1) & 1);
         __syncthreads();
