@@ -195,7 +195,16 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
 #pragma unroll
     for (int j = 0; j < STAGES; ++j) {
       if (i + j < n64) {  // the same for the whole wave, and a scalar branch
-        if (i + j + STAGES - 1 < n64) load_step((j + STAGES - 1) % STAGES, i + j + STAGES - 1);
+        if constexpr (STAGES == 4) {
+          // two steps asked for together: a row's 256 contiguous bytes reach the memory
+          // close in time
+          if ((j & 1) == 0) {
+            if (i + j + 2 < n64 && i + j + 2 >= STAGES - 1) load_step((j + 2) % STAGES, i + j + 2);
+            if (i + j + 3 < n64) load_step((j + 3) % STAGES, i + j + 3);
+          }
+        } else {
+          if (i + j + STAGES - 1 < n64) load_step((j + STAGES - 1) % STAGES, i + j + STAGES - 1);
+        }
         mma_step(j);
       }
     }
