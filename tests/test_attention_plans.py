@@ -37,3 +37,37 @@ def test_single_tokens_split_until_the_chip_is_full():
     assert decode_splits(64, 8, 640, 4, 0) == 1
     assert decode_splits(1, 8, 100000, 8, 0) == 32
     assert decode_splits(1, 8, 100000, 8, 64) <= 2  # a window of 64 keys is a handful of blocks
+
+
+def test_row_counts_choose_how_norms_and_products_meet():
+    import torch
+
+    from kvcore_amd.ops import library as ops
+
+    bf16, f32 = torch.bfloat16, torch.float32
+    # a width the kernels for a few dozen rows take: the fold stops at 8 rows
+    assert ops.rows_fusable(1, bf16, 4096) and ops.rows_fusable(8, bf16, 4096)
+    assert not ops.rows_fusable(9, bf16, 4096) and ops.rows_sinkable(9, bf16, 4096)
+    assert ops.rows_sinkable(64, bf16, 4096) and not ops.rows_sinkable(65, bf16, 4096)
+    # a narrow model keeps the fold up to 16 rows
+    assert ops.rows_fusable(16, bf16, 128) and not ops.rows_sinkable(16, bf16, 128)
+    assert ops.rows_sinkable(17, bf16, 128)
+    # never both, and float32 neither
+    for rows in range(0, 80):
+        for width in (96, 512, 4096):
+            assert not (ops.rows_fusable(rows, bf16, width) and ops.rows_sinkable(rows, bf16, width))
+            assert not ops.rows_fusable(rows, f32, width) and not ops.rows_sinkable(rows, f32, width)
+
+
+def test_slices_along_k_stay_within_the_bound_a_block_reserves_for():
+    from kvcore_amd.ops import library as ops
+
+    for N in (64, 200, 2048, 4096, 8192, 14336, 128256):
+        bound = ops.mid_slices_bound(N)
+        assert 1 <= bound <= 64
+        for K in (512, 1024, 4096, 14336, 28672, 65536):
+            s = ops.mid_slices(N, K)
+            assert 1 <= s <= bound, (N, K, s, bound)
+            assert s <= K // 512
+    assert ops.mid_slices(4096, 4096) == 4 and ops.mid_slices(128256, 4096) == 1
+    assert ops.mid_slices(4096, 520) == 0  # a K the kernel does not take
