@@ -56,7 +56,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
                                    int M, int N, int K, int64_t lda, int64_t ldc, int k_per_wave,
                                    const SkinnyExtras ex) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
-  extern __shared__ float red[];  // [waves - 1][RT * NT][64][4]
+  extern __shared__ float red[];  // [waves - 1][RT * NT][64][4], then 16 row scales and [16][256] parts of their sums if FOLD & 1
   // wave-uniform values are made scalar on purpose: a condition on them becomes a scalar
   // branch, and matrix instructions are only ever skipped by branches (they do not honour
   // the lane mask that a vector condition would leave)
@@ -146,16 +146,35 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
   // (Loads without a branch around them would let the waits count them exactly and keep
   // all STAGES steps in flight; measured inside a decode step that is slower than this form,
   // whose waits drain more often but which needs fewer registers and so runs more waves.)
+  // The rows' scale factors.  Where a row's parts fit one 16-byte load a lane, every wave
+  // asks for the parts of its share of the rows now, before its weights, straight into LDS
+  // (no registers wait for them), and adds them up only after its walk along K: loads
+  // complete in the order of their issue, so by then they have long arrived.
+  float* scale_lds = red + static_cast<int64_t>(waves - 1) * (RT * NT) * 256;  // [16] row scales,
+  float* parts_lds = scale_lds + 16;                                           // then [16][256] parts
+  bool ss_late = false;
+  if constexpr ((FOLD & 1) != 0 && NT == 1) {
+    // (one or two rows cost the old way nothing: a single round of loads while the weights come)
+    ss_late = M > 2 && ex.in_parts % 4 == 0 && ex.in_parts <= 256 && (reinterpret_cast<uintptr_t>(ex.in_ss) & 15) == 0;
+    if (ss_late) {
+      for (int t = wave; t < M; t += waves) {  // scalar
+        if (4 * lane < ex.in_parts)
+          __builtin_amdgcn_global_load_lds(
+              (const __attribute__((address_space(1))) void*)(ex.in_ss + static_cast<int64_t>(t) * ex.in_parts + 4 * lane),
+              (__attribute__((address_space(3))) void*)(parts_lds + t * 256), 16, 0, 0);
+      }
+    }
+  }
   int k = k_begin;
 #pragma unroll
   for (int st = 0; st < STAGES - 1; ++st)
     if (st < n64) load_step(st, st);
-  // The rows' scale factors, worked out by the wave that will need them at the end while its
+  // Otherwise they are worked out by the wave that will need them at the end while its
   // first weight loads are on their way, four tokens at a time (more would cost registers and
   // with them waves in flight).  Token by token the wave reads the row's parts (four a lane)
   // and adds them up in the fixed order of a butterfly, so the result does not depend on
   // anything but the parts.
-  if ((FOLD & 1) && wave == 0) {
+  if ((FOLD & 1) && wave == 0 && !ss_late) {
     const bool vec = (ex.in_parts % 4 == 0) && ((reinterpret_cast<uintptr_t>(ex.in_ss) & 15) == 0);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -239,6 +258,18 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
         acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt], b[nt], acc[rt][nt], 0, 0, 0);
   }
 
+  if constexpr ((FOLD & 1) != 0 && NT == 1) {
+    if (ss_late) {
+      // the wave's own loads into LDS have all landed once its load counter is at zero
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      for (int t = wave; t < M; t += waves) {
+        f32x4_t v = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if (4 * lane < ex.in_parts) v = *reinterpret_cast<const f32x4_t*>(parts_lds + t * 256 + 4 * lane);
+        const float total = wave_sum((v[0] + v[1]) + (v[2] + v[3]));
+        if (lane == 0) scale_lds[t] = rsqrtf(total / ex.in_width + ex.in_eps);
+      }
+    }
+  }
   constexpr int TILES = RT * NT;
   if (wave > 0) {
 #pragma unroll
@@ -250,6 +281,9 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
   }
   __syncthreads();
   if (wave != 0) return;
+  if constexpr ((FOLD & 1) != 0 && NT == 1) {
+    if (ss_late && tok_ok[0]) row_scale[0] = scale_lds[col];
+  }
   for (int w = 1; w < waves; ++w) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
@@ -355,7 +389,8 @@ void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M
   // steps in flight by what fits in registers beside the accumulators
   constexpr int STAGES = (RT + NT <= 5) ? 4 : ((RT + NT <= 6) ? 3 : 2);
   constexpr int MAXW = (RT >= 2) ? 4 : 8;
-  const size_t lds = static_cast<size_t>(waves - 1) * RT * NT * 64 * 4 * sizeof(float);
+  const size_t lds = static_cast<size_t>(waves - 1) * RT * NT * 64 * 4 * sizeof(float) +
+                     (ex.in_ss != nullptr ? (16 + 16 * 256) * sizeof(float) : 0);
   const int rows_per_block = GATED ? 16 : 16 * RT;
   const dim3 grid((N + rows_per_block - 1) / rows_per_block), block(waves * 64);
   const int fold = (ex.in_ss != nullptr ? 1 : 0) | (ex.residual != nullptr ? 2 : 0);
