@@ -203,22 +203,26 @@ def main() -> int:
                           "frac": round(prefill_flops(cfg, args.long_prompt) / sec / PEAK_FLOPS[args.dtype], 4)}))
         return 0
     if args.mixed:
-        lens = [rng.randrange(16, 2049) for _ in range(64)]
         engine.scheduler.config = SchedulerConfig(
             max_num_seqs=max_seqs, max_num_scheduled_tokens=PREFILL_TOKENS, max_num_partial_prefills=max_seqs,
             max_long_partial_prefills=max_seqs, long_prefill_token_threshold=512)
-        for n in lens:
-            new_request(n, 128)
-        torch.cuda.synchronize()
-        t_start = time.perf_counter()
-        steps = 0
-        while engine.has_unfinished_requests():
-            engine.step()
-            steps += 1
-        torch.cuda.synchronize()
-        sec = time.perf_counter() - t_start
+        lens = [rng.randrange(16, 2049) for _ in range(64)]
+        runs = []
+        for _ in range(2):  # the first pass also captures the graphs of the decode steps it meets
+            for n in lens:
+                new_request(n, 128)
+            torch.cuda.synchronize()
+            t_start = time.perf_counter()
+            steps = 0
+            while engine.has_unfinished_requests():
+                engine.step()
+                steps += 1
+            torch.cuda.synchronize()
+            runs.append(time.perf_counter() - t_start)
+        sec = runs[1]
         print(json.dumps({"workload": "mixed: 64 requests, prompts U[16,2048], portions of 512, 128 new tokens",
-                          "model": model_name, "dtype": args.dtype, "seconds": round(sec, 4), "steps": steps,
+                          "model": model_name, "dtype": args.dtype, "seconds": round(sec, 4),
+                          "first_pass_seconds": round(runs[0], 4), "steps": steps,
                           "prompt_tokens": sum(lens), "generated_tokens": 64 * 128,
                           "generated_tokens_per_s": round(64 * 128 / sec, 1),
                           "total_tokens_per_s": round((sum(lens) + 64 * 128) / sec, 1)}))
