@@ -898,7 +898,8 @@ def test_sample_follows_the_probabilities_and_top_k_top_p_vectors(ops):
     assert got == {0, 1}
 
 
-@pytest.mark.parametrize("M,H,I", [(1, 64, 48), (8, 4096, 1024), (16, 136, 200), (5, 4104, 88)])
+@pytest.mark.parametrize("M,H,I", [(1, 64, 48), (8, 4096, 1024), (16, 136, 200), (5, 4104, 88),
+                                   (8, 2048, 512), (3, 512, 64)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_norms_folded_into_the_products_around_them(ops, M, H, I, with_bias):
     """residual += x1 W1^T; x2 = rmsnorm(residual) * gain; y = silu(x2 Wg^T) * (x2 Wu^T), once
