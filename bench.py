@@ -69,6 +69,7 @@ def parse_args():
     p.add_argument("--long-prompt", type=int, default=0, metavar="N",
                    help="time to the first token of one N-token prompt, in portions of 2,048 "
                         "tokens; prints its own line")
+    p.add_argument("--page-size", type=int, default=PAGE_SIZE, help="tokens a cache page")
     p.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     p.add_argument("--only-prefill", action="store_true",
                    help="run only the 2,048-token prefill (for profiling); prints its own line")
@@ -124,14 +125,14 @@ def main() -> int:
           f"{model.num_param_bytes() / 2**30:.2f} GiB", file=sys.stderr, flush=True)
 
     max_seqs = 64
-    pages_per_seq = -(-(PREFILL_TOKENS + NEW_TOKENS + prompt_len) // PAGE_SIZE)
+    pages_per_seq = -(-(PREFILL_TOKENS + NEW_TOKENS + prompt_len) // args.page_size)
     if args.long_prompt:
-        max_seqs, pages_per_seq = 2, -(-(args.long_prompt + 16) // PAGE_SIZE)
+        max_seqs, pages_per_seq = 2, -(-(args.long_prompt + 16) // args.page_size)
     engine = EngineCore(KVCoreConfig(
         model_config=ModelConfig(model=".", dtype=args.dtype,
                                  max_model_len=max(CONTEXT_LEN, args.long_prompt + 16)),
         load_config=LoadConfig(load_format="random", seed=0),
-        cache_config=CacheConfig(block_size=PAGE_SIZE, num_gpu_blocks=max_seqs * pages_per_seq + 1),
+        cache_config=CacheConfig(block_size=args.page_size, num_gpu_blocks=max_seqs * pages_per_seq + 1),
         scheduler_config=SchedulerConfig(max_num_seqs=max_seqs, max_num_scheduled_tokens=PREFILL_TOKENS,
                                          max_num_partial_prefills=max_seqs,
                                          max_long_partial_prefills=max_seqs),
@@ -248,7 +249,7 @@ def main() -> int:
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"],
             "vocab": cfg["vocab_size"], "global_batch": args.batch, "seq_len": CONTEXT_LEN,
-            "prompt_len": prompt_len, "new_tokens": NEW_TOKENS, "page_size": PAGE_SIZE,
+            "prompt_len": prompt_len, "new_tokens": NEW_TOKENS, "page_size": args.page_size,
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single-gpu",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
