@@ -548,7 +548,8 @@ def mid_slices(N: int, K: int) -> int:
     return int(load().kvc_gemm_mid_slices(N, K))
 
 
-def _mid_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+def mid_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``gemm_mid`` takes these operands (K a multiple of 512, aligned rows)."""
     return (x.shape[1] % 512 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and w.is_contiguous()
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
@@ -563,7 +564,7 @@ def gemm_mid(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias: t
     N = w.shape[0] // 2 if mode == 1 else w.shape[0]
     if w.shape[1] != K or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not x.is_cuda:
         raise KernelError("gemm_mid: operands must be bfloat16 GPU tensors with matching K")
-    if not _mid_operands_ok(x, w):
+    if not mid_operands_ok(x, w):
         raise KernelError("gemm_mid: K must be a multiple of 512 and the operands aligned")
     if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != w.shape[0]):
         raise KernelError("gemm_mid: bias must be bfloat16, one value per weight row")
@@ -613,7 +614,7 @@ def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.
     # long (8192 x 8192), and slower for narrow outputs and long K (8192 x 28672: 139 against
     # 107 us at 64 rows; 4096 x 4096: 19 against 12)
     ours = N < 8192 or K > 8192
-    if ours and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _mid_operands_ok(x, w) and N % 8 == 0:
+    if ours and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and mid_operands_ok(x, w) and N % 8 == 0:
         slices = mid_slices(N, K)
         if sink.slices.numel() < slices * M * N:
             raise KernelError("linear: the sink's workspace is too small")
@@ -642,7 +643,7 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
         raise KernelError("linear_silu_mul: shapes do not match")
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and x.is_cuda and _skinny_operands_ok(x, w)
-            and (M <= FOLD_ROWS or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and not _mid_operands_ok(x, w)))):
+            and (M <= FOLD_ROWS or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and not mid_operands_ok(x, w)))):
         if M == 0:
             return
         if bias is not None and (bias.dtype != torch.bfloat16 or bias.shape != (2 * I,)):
@@ -652,7 +653,7 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
             M, I, K, x.stride(0), out.stride(0), _stream()), "kvc_gemm_skinny_silu_mul_bf16")
         return
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
-            and x.is_cuda and FOLD_ROWS < M <= MID_ROWS and _mid_operands_ok(x, w)
+            and x.is_cuda and FOLD_ROWS < M <= MID_ROWS and mid_operands_ok(x, w)
             and out.stride(1) == 1):
         # 9 to 64 rows: the waves of a block share the rows through LDS
         gemm_mid(out, x, w, bias, mode=1)

@@ -45,9 +45,16 @@ class OutputHead(Part):
             ops.linear(logits, hidden_rows, w)
             return
         S = hidden_rows.shape[0]
-        if self.hidden_size % 8 == 0 and (S <= 8 or (S <= ops.SKINNY_PREFERRED_ROWS
-                                                      and self.vocab_size < 65536)):
+        # measured at 128256 x 4096: the few-row kernel wins up to 12 rows, the kernel that
+        # shares the rows through LDS from 24 on (215 against 231 us at 64 rows), the vendor
+        # product with a conversion afterwards in between and beyond 64
+        if self.hidden_size % 8 == 0 and (S <= 12 or (S <= ops.SKINNY_PREFERRED_ROWS
+                                                       and self.vocab_size < 65536)):
             ops.linear(logits, hidden_rows, w)  # float32 sums are stored without rounding
+            return
+        if ops.SKINNY_PREFERRED_ROWS < S <= ops.MID_ROWS and ops.mid_operands_ok(hidden_rows, w) \
+                and logits.stride(1) == 1:
+            ops.gemm_mid(logits, hidden_rows, w, mode=0)  # float32 sums, stored as they are
             return
         low = ctx.buffers.get("head_logits_dt", S, self.vocab_size, hidden_rows.dtype)
         ops.linear(low, hidden_rows, w)
