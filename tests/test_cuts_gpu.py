@@ -404,3 +404,45 @@ def test_steps_of_a_few_dozen_rows_on_a_wide_model(tmp_path, monkeypatch):
     rms = float(torch.cat([e.flatten() for e in expect.values()]).pow(2).mean().sqrt())
     assert 0.4 < rms < 0.55
     compare(got, expect, torch.bfloat16, logit_rms=rms)
+
+
+def test_layer_sizes_of_the_8b_model(tmp_path):
+    """One layer with the widths of Llama-3-8B (4096 wide, 32 heads of 128 over 8 kv heads,
+    14336 in the feed-forward) and a small vocabulary, against the plain implementation in
+    float32: the shapes that decide which kernel runs are the real ones.  Prompts whole, then
+    12 rows together (the kernels that share the rows through LDS), then 3 (the few-row
+    kernels with the norms folded in), through graphs where the runner uses them."""
+    config = {
+        "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 1,
+        "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+        "intermediate_size": 14336, "vocab_size": 384, "rope_theta": 500000.0,
+        "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                         "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
+        "tie_word_embeddings": False, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192,
+        "hidden_act": "silu",
+    }
+    folder = make_model_dir(tmp_path / "wide8b", config, seed=5)
+    cfg, weights = plain.load_model_folder(folder)
+    n_req, tail = 12, 6
+    seqs = {f"r{i}": random_tokens(20 + 3 * i + tail, cfg["vocab_size"], seed=900 + i) for i in range(n_req)}
+    total = sum(-(-len(t) // 64) * 64 for t in seqs.values())
+    session = session_for(folder, torch.bfloat16, 16, max_tokens=total, max_num_seqs=16)
+    expect = {rid: plain.llama_forward(cfg, weights, t, dtype=torch.float32).double() for rid, t in seqs.items()}
+    ids = list(seqs)
+    steps, k = [], 0
+    for i in range(0, n_req, 4):
+        steps.append({"step": k, "end": [], "entries": [
+            {"id": r, "tokens": seqs[r][:len(seqs[r]) - tail], "want": [0, len(seqs[r]) - tail - 1]}
+            for r in ids[i:i + 4]]})
+        k += 1
+    fed = {r: len(seqs[r]) - tail for r in ids}
+    for j in range(tail):
+        live = ids if j < 3 else ids[:3]
+        steps.append({"step": k, "end": ids[3:] if j == 2 else [], "entries": [
+            {"id": r, "tokens": [seqs[r][fed[r]]], "want": [0]} for r in live]})
+        k += 1
+        for r in live:
+            fed[r] += 1
+    got = collect(session, steps)
+    rms = float(torch.cat([e.flatten() for e in expect.values()]).pow(2).mean().sqrt())
+    compare(got, expect, torch.bfloat16, logit_rms=rms)
