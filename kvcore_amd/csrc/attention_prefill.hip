@@ -21,6 +21,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "attention_combine.h"
 #include "device_utils.h"
 #include "kvcore_hip.h"
@@ -59,7 +61,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     const int32_t* __restrict__ table, int table_stride, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int num_reqs, int nh,
     int nkv, int page_size, int num_pages, float scale_log2e, int window,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, int single) {
   constexpr int NJ = D / 16;
   constexpr int NC = D / 32;
   constexpr int KROW = D + 8;  // padded K row in LDS (elements)
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     for (int r = 0; r < num_reqs; ++r) {
       const int b = q_start[r], e = q_start[r + 1];
       const int tiles_r = (e - b + bq - 1) / bq;
-      const int pairs_r = (tiles_r + 1) / 2;
+      const int pairs_r = single ? tiles_r : (tiles_r + 1) / 2;
       if (idx < pairs_r) {
         req = r;
         pair = idx;
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   const int32_t* row_table = table + static_cast<int64_t>(slots[req]) * table_stride;
   for (int turn = 0; turn < 2; ++turn) {
   const int tile = (turn == 0) ? n_tiles - 1 - pair : pair;
-  if (turn == 1 && tile == n_tiles - 1 - pair) break;  // the middle tile was the first turn
+  if (turn == 1 && (single || tile == n_tiles - 1 - pair)) break;  // the middle tile was the first turn
   if (turn == 1) __syncthreads();  // the first turn's last tile has been consumed by every wave
   const int t0 = q_begin + tile * bq;
   const int t_end = (t0 + bq < q_end) ? t0 + bq : q_end;
@@ -460,11 +462,11 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
                       const bf16_t* v_cache, const int32_t* table, int table_stride,
                       const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                       int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
-                      float* part_o, float* part_ml, int nsplit, hipStream_t stream) {
+                      float* part_o, float* part_ml, int nsplit, int single, hipStream_t stream) {
   const int g = nh / nkv;
   const int bq = (64 * CT) / g;
   // every request may end in a ragged tile and have an odd number of tiles
-  const int max_pairs = ((T + bq - 1) / bq + R) / 2 + R;
+  const int max_pairs = single ? (T + bq - 1) / bq + R : ((T + bq - 1) / bq + R) / 2 + R;
   constexpr int lds_bytes = 2 * tile_bytes<D>();
   static const hipError_t attr = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&prefill_attention_kernel<D, CT>),
@@ -473,7 +475,7 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
   hipLaunchKernelGGL((prefill_attention_kernel<D, CT>), dim3(max_pairs, nkv, nsplit), dim3(kWaves * 64),
                      lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                      q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, part_o,
-                     part_ml);
+                     part_ml, single);
   if (nsplit > 1) return launch_attention_combine(out, part_o, part_ml, static_cast<int64_t>(T) * nh, D, nsplit, stream);
   return kvc_check_launch("kvc_prefill_attention");
 }
@@ -485,18 +487,43 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
                    int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
                    float* part_o, float* part_ml, int nsplit, hipStream_t stream) {
   const int g = nh / nkv;
-  // Tiles of 128 query rows stage each key tile for twice the rows, tiles of 64 make twice
-  // the blocks: the larger ones once their blocks alone give every compute unit two, and
-  // whenever the keys are split (the caller splits until there are blocks enough).
-  const int bq2 = 128 / g > 0 ? 128 / g : 1;
-  const int64_t pairs2 = static_cast<int64_t>(((T + bq2 - 1) / bq2 + 1) / 2) * nkv;
-  if (pairs2 >= 512 || nsplit > 1 || g > 64)
+  // A compute unit holds two blocks.  Tiles of 64 query rows, two a block one after the other
+  // (a late and an early one), are the fastest as long as all their blocks find room at once;
+  // more rows than that take tiles of 128 rows, which stage each key tile for twice the rows
+  // (and so does a launch that splits the keys, unless its rows are very few: its caller splits
+  // until there are blocks enough).  Few rows take one tile of 64 a block, for twice the blocks.  Measured at 32
+  // heads over 8 kv heads of 128: 1,024 tokens 43 against 47 us, 2,048 tokens 94 (pairs of
+  // 64) against 113 (pairs of 128), 3,072 tokens 165 (pairs of 128) against 217.
+  // (every request but one may add a ragged tile)
+  const int bq1 = 64 / g > 0 ? 64 / g : 1;
+  const int tiles1 = (T + bq1 - 1) / bq1 + (R - 1);
+  const int64_t pairs1 = static_cast<int64_t>((tiles1 + 1) / 2) * nkv;
+  const int64_t small_tiles = static_cast<int64_t>(tiles1) * nkv;
+  int ct = 1, single = 0;
+  if (g > 64) {
+    ct = 2;
+  } else if (nsplit > 1) {
+    // very few rows: small tiles one a block reach the blocks wanted with a quarter of the
+    // splits (128 rows at 1,024 keys: 21 against 39 us)
+    if (small_tiles <= 128) single = 1; else ct = 2;
+  } else if (pairs1 > 512) {
+    ct = 2;
+  } else if (pairs1 <= 256) {
+    single = 1;
+  }
+  // KVC_PREFILL_MODE = 1p | 1s | 2p overrides the choice for tuning
+  static const char* mode = getenv("KVC_PREFILL_MODE");
+  if (mode && (mode[0] == '1' || mode[0] == '2')) {
+    ct = mode[0] == '2' ? 2 : 1;
+    single = mode[1] == 's';
+  }
+  if (ct == 2)
     return launch_prefill_ct<D, 2>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                                    q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window,
-                                   part_o, part_ml, nsplit, stream);
+                                   part_o, part_ml, nsplit, single, stream);
   return launch_prefill_ct<D, 1>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                                  q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window,
-                                 part_o, part_ml, nsplit, stream);
+                                 part_o, part_ml, nsplit, single, stream);
 }
 
 }  // namespace

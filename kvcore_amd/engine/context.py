@@ -58,13 +58,16 @@ class StepBuffers:
     """Named device buffers that live across steps, so a step allocates nothing once
     the largest batch has been seen.  ``get`` returns a view of the first ``rows`` rows.
 
-    Buffers indexed by token are allocated for ``token_capacity`` rows at once.  A buffer
-    that still has to grow is replaced by a new tensor; ``on_grow`` is then called first,
-    because a captured graph holds the old address."""
+    Buffers indexed by token are allocated for ``token_capacity`` rows at once, buffers with
+    a row per request that samples for ``seq_capacity`` rows (``reserve`` of ``get``).  A
+    buffer that still has to grow is replaced by a new tensor; ``on_grow`` is then called
+    first, because a captured graph holds the old address."""
 
-    def __init__(self, device: torch.device, token_capacity: int = 0, on_grow=None) -> None:
+    def __init__(self, device: torch.device, token_capacity: int = 0, on_grow=None,
+                 seq_capacity: int = 0) -> None:
         self.device = device
         self.token_capacity = token_capacity
+        self.seq_capacity = seq_capacity
         self.on_grow = on_grow
         self._store: dict[str, torch.Tensor] = {}
         self.frozen = False

@@ -127,7 +127,8 @@ class ModelRunner:
             if runner is not None:
                 runner._drop_graphs()
 
-        self.buffers = StepBuffers(self.device, token_capacity=max_num_tokens, on_grow=drop_graphs)
+        self.buffers = StepBuffers(self.device, token_capacity=max_num_tokens, on_grow=drop_graphs,
+                                   seq_capacity=max_num_seqs)
 
         # host mirror of what each slot's table rows hold: (request id, entries synced,
         # leading entries nulled) per group

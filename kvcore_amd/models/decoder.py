@@ -183,8 +183,11 @@ class DecoderModel:
                        num_rows: int) -> torch.Tensor:
         """float32 ``[S, V]`` at the flattened token indices ``rows[:S]``."""
         H, V = self.spec.hidden_size, self.spec.vocab_size
-        picked = ctx.buffers.get("head_rows", num_rows, H, self.dtype)
+        # a row per request that samples, as a rule: room for all of them at once, so that a
+        # batch that fills up step by step does not make these grow (and drop the graphs)
+        room = ctx.buffers.seq_capacity
+        picked = ctx.buffers.get("head_rows", num_rows, H, self.dtype, reserve=room)
         ops.gather_rows(picked, hidden, rows[:num_rows])
-        logits = ctx.buffers.get("logits", num_rows, V, torch.float32)
+        logits = ctx.buffers.get("logits", num_rows, V, torch.float32, reserve=room)
         self.head.forward(logits, picked, ctx)
         return logits

@@ -26,26 +26,40 @@ def prefill_split_rows(nkv: int, g: int) -> int:
 
 
 PREFILL_TARGET_BLOCKS = 512
+PREFILL_FEW_TILES = 128     # up to so many small tiles, splits go with small tiles
 PREFILL_MIN_KEYS = 256      # for steps of few tokens, whose partial results are small
 PREFILL_MIN_KEYS_MOST = 1024
 PREFILL_MAX_SPLITS = 32
 
 
-def prefill_splits(T: int, nkv: int, g: int, max_query_len: int, max_seq_len: int, window: int) -> int:
+def prefill_splits(T: int, nkv: int, g: int, max_query_len: int, max_seq_len: int, window: int,
+                   num_reqs: int = 1) -> int:
     """How many blocks share the keys of one tile of query rows in the kernel for portions
-    of prompts.  One, unless the step has too few tiles of 128 query rows to give every
-    compute unit two blocks; then as many as make up for it, while every block still has
-    keys enough to walk to be worth its partial results: a few hundred, a thousand for steps
-    of thousands of tokens (a row sees ``max_seq_len`` keys at most and, under the causal
-    mask, about half a portion fewer on average)."""
-    rows_tokens = max(128 // g, 1)
-    blocks = ((-(-T // rows_tokens)) + 1) // 2 * nkv
-    if blocks >= PREFILL_TARGET_BLOCKS:
-        return 1
+    of prompts.  A compute unit holds two of its blocks, so a launch wants some 512.  The
+    kernel has tiles of 64 rows (one or two a block) and of 128 (two a block, cheaper per
+    key); with splits it takes the small tiles one a block for very few rows and the large
+    ones otherwise (`launch_prefill` in csrc/attention_prefill.hip, which must agree with
+    this on where "very few" ends).  Measured on the 8B shape: splits pay when the rows are
+    few and every block still has a few hundred keys to walk, a thousand for steps of a
+    thousand tokens (a row sees ``max_seq_len`` keys at most and, under the causal mask,
+    about half a portion fewer on average).  Every request but one may add a ragged tile."""
+    small_tokens = max(64 // g, 1)
+    small_tiles = (-(-T // small_tokens) + num_reqs - 1) * nkv  # blocks of one small tile each
     keys = max_seq_len - min(T, max_query_len) // 2
     if window > 0:
-        keys = min(keys, window + rows_tokens)
-    min_keys = min(max(T // 2, PREFILL_MIN_KEYS), PREFILL_MIN_KEYS_MOST)
+        keys = min(keys, window + 2 * small_tokens)
+    if small_tiles <= PREFILL_FEW_TILES:
+        return max(1, min(-(-PREFILL_TARGET_BLOCKS // small_tiles), keys // PREFILL_MIN_KEYS, PREFILL_MAX_SPLITS))
+    if small_tiles <= PREFILL_TARGET_BLOCKS:
+        if small_tiles == PREFILL_TARGET_BLOCKS:
+            return 1  # one small tile a block fills the chip as it is
+        min_keys = min(max(T, PREFILL_MIN_KEYS), PREFILL_MIN_KEYS_MOST)
+    else:
+        min_keys = min(max(T // 2, PREFILL_MIN_KEYS), PREFILL_MIN_KEYS_MOST)
+    rows_tokens = max(128 // g, 1)
+    blocks = ((-(-T // rows_tokens)) + num_reqs) // 2 * nkv
+    if blocks >= PREFILL_TARGET_BLOCKS:
+        return 1
     return max(1, min(-(-PREFILL_TARGET_BLOCKS // blocks), keys // min_keys, PREFILL_MAX_SPLITS))
 
 
@@ -140,9 +154,14 @@ class PagedAttention(Mixer):
             nsplit = decode_splits(T, self.num_kv_heads, ctx.max_seq_len, waves, self.window)
             part_o = part_ml = None
             if nsplit > 1:
+                # tokens x splits is at most the blocks wanted per kv head plus the tokens: room
+                # for the largest at once, since a buffer that grows drops the graphs
+                most = (DECODE_TARGET_BLOCKS // self.num_kv_heads + 1 + max(T, ctx.buffers.seq_capacity)) \
+                    * self.num_heads
                 part_o = ctx.buffers.get("attn_part_o", T * self.num_heads * nsplit, self.head_dim,
-                                         torch.float32)
-                part_ml = ctx.buffers.get("attn_part_ml", T * self.num_heads * nsplit, 2, torch.float32)
+                                         torch.float32, reserve=most)
+                part_ml = ctx.buffers.get("attn_part_ml", T * self.num_heads * nsplit, 2, torch.float32,
+                                          reserve=most)
             ops.decode_attention(attn, qkv, k_cache, v_cache, nsplit=nsplit, part_o=part_o,
                                  part_ml=part_ml, cos=cos, sin=sin, rot_dim=rot_dim,
                                  interleaved=interleaved, write_kv=call.write_cache,
@@ -166,7 +185,7 @@ class PagedAttention(Mixer):
                 # block, and several blocks per tile where few rows meet many keys
                 T = ctx.num_tokens
                 nsplit = prefill_splits(T, self.num_kv_heads, self.num_heads // self.num_kv_heads,
-                                        ctx.max_query_len, ctx.max_seq_len, self.window)
+                                        ctx.max_query_len, ctx.max_seq_len, self.window, ctx.num_reqs)
                 part_o = part_ml = None
                 if nsplit > 1:
                     # asked for at their largest at once: a buffer that grows drops the graphs

@@ -56,6 +56,7 @@ class OutputHead(Part):
                 and logits.stride(1) == 1:
             ops.gemm_mid(logits, hidden_rows, w, mode=0)  # float32 sums, stored as they are
             return
-        low = ctx.buffers.get("head_logits_dt", S, self.vocab_size, hidden_rows.dtype)
+        low = ctx.buffers.get("head_logits_dt", S, self.vocab_size, hidden_rows.dtype,
+                              reserve=ctx.buffers.seq_capacity)
         ops.linear(low, hidden_rows, w)
         ops.to_float(logits, low)
