@@ -47,14 +47,14 @@ __device__ __forceinline__ s16x4_t pack_bf16x4(const float* p) {
 }
 
 constexpr int kWaves = 4;
-constexpr int kKeyBlocks = 4;  // 16-key blocks per LDS tile
 
-template <int D>
+// KB: 16-key blocks per LDS tile
+template <int D, int KB>
 constexpr int tile_bytes() {
-  return kKeyBlocks * 16 * (D + 8) * 2 + kKeyBlocks * D * 16 * 2;  // K rows padded, then V
+  return KB * 16 * (D + 16) * 2 + KB * D * 16 * 2;  // K rows padded, then V
 }
 
-template <int D, int CT>
+template <int D, int CT, int KB>
 __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -62,11 +62,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int num_reqs, int nh,
     int nkv, int page_size, int num_pages, float scale_log2e, int window,
     float* __restrict__ part_o, float* __restrict__ part_ml, int single) {
+  constexpr int kKeyBlocks = KB;
   constexpr int NJ = D / 16;
   constexpr int NC = D / 32;
-  constexpr int KROW = D + 8;  // padded K row in LDS (elements)
+  // padded K row in LDS (elements): with 32 bytes of padding the operand reads (16 rows x 4
+  // pieces of 16 bytes a wave) meet no bank conflict; with 16 they took 1.45 times as long
+  constexpr int KROW = D + 16;
   constexpr int K_ELEMS = kKeyBlocks * 16 * KROW;
-  constexpr int TILE_ELEMS = tile_bytes<D>() / 2;
+  constexpr int TILE_ELEMS = tile_bytes<D, KB>() / 2;
   extern __shared__ __attribute__((aligned(16))) bf16_t tiles[];  // two tiles: [K | V] each
 
   const int g = nh / nkv;
@@ -232,7 +235,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
         if constexpr (D == 128) {
           base = vpage[i];
         } else {
-          base = (tid < 128) ? vpage[2 * i] : vpage[2 * i + 1];
+          base = (tid < 128) ? vpage[i] : vpage[2 + i];
         }
         vreg[i] = (base >= 0) ? *reinterpret_cast<const uint4*>(v_cache + base + v_off[i])
                               : make_uint4(0u, 0u, 0u, 0u);
@@ -256,14 +259,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
-      // piece (i*256 + tid) of the tile: key block, then row of the head, then half of 16 keys
-      const int kbi = (D == 128) ? i : 2 * i + (tid >> 7);
+      // this thread's pieces: both key blocks of a pair, one row of the head, one half of 16 keys
+      const int kbi = (D == 128) ? i : 2 * (tid >> 7) + i;
       const int half = tid & 1;
       int64_t base;
       if constexpr (D == 128) {
         base = vpage[i];
       } else {
-        base = (tid < 128) ? vpage[2 * i] : vpage[2 * i + 1];
+        base = (tid < 128) ? vpage[i] : vpage[2 + i];
       }
       uint4 val = make_uint4(0u, 0u, 0u, 0u);
       const int key0 = (kb0 + kbi) * 16 + half * 8;
@@ -282,32 +285,30 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     }
   };
   // Registers to LDS.  K: [key][KROW].  V: [pair of key blocks][16-row group j][quad][row in
-  // group][8 keys], the eight keys being 4*quad .. +4 of the pair's first block and then of
-  // its second, so that the 64 lanes of an A-operand read (lane = quad*16 + row) touch 1024
-  // consecutive bytes.
+  // group, flipped by 8 for quads 2 and 3][8 keys], the eight keys being 4*quad .. +4 of the
+  // pair's first block and then of its second, so that the 64 lanes of an A-operand read
+  // (lane = quad*16 + row) touch 1024 consecutive bytes.
   auto store_tile = [&](int buf) {
     bf16_t* k_lds = tiles + buf * TILE_ELEMS;
     bf16_t* v_lds = k_lds + K_ELEMS;
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i)
       *reinterpret_cast<uint4*>(k_lds + (i * ROWS_PER_STEP + k_row0) * KROW + k_piece * 8) = kreg[i];
+    // A thread holds the same eight keys of both key blocks of a pair (head size 128: two
+    // pairs), so it stores whole 16-byte slots: [4 keys of the first block | 4 of the second]
+    // for quad 2*half and for quad 2*half + 1.  The row within the 16-row group is flipped by
+    // 8 for quads 2 and 3, so that the 16 lanes that store together (8 rows x 2 halves) hit
+    // 16 different slots; the reads flip it back.
 #pragma unroll
-    for (int i = 0; i < V_PER_THREAD; ++i) {
-      int kbi, rem;
-      if constexpr (D == 128) {
-        kbi = i;
-        rem = tid;
-      } else {
-        kbi = 2 * i + (tid >> 7);
-        rem = tid & 127;
-      }
+    for (int pr = 0; pr < V_PER_THREAD / 2; ++pr) {
+      const int rem = (D == 128) ? tid : (tid & 127);
+      const int pair = (D == 128) ? pr : (tid >> 7);
       const int drow = rem >> 1;
       const int half = rem & 1;
-      // keys 8*half .. +4 belong to quad 2*half, the next four to quad 2*half + 1
-      bf16_t* dst = v_lds + (((((kbi >> 1) * NJ + (drow >> 4)) * 4 + 2 * half) * 16 + (drow & 15)) * 8) +
-                    4 * (kbi & 1);
-      *reinterpret_cast<uint2*>(dst) = make_uint2(vreg[i].x, vreg[i].y);
-      *reinterpret_cast<uint2*>(dst + 16 * 8) = make_uint2(vreg[i].z, vreg[i].w);
+      const uint4 a = vreg[2 * pr], b = vreg[2 * pr + 1];
+      bf16_t* dst = v_lds + (((pair * NJ + (drow >> 4)) * 4 + 2 * half) * 16 + ((drow & 15) ^ (8 * half))) * 8;
+      *reinterpret_cast<uint4*>(dst) = make_uint4(a.x, a.y, b.x, b.y);
+      *reinterpret_cast<uint4*>(dst + 16 * 8) = make_uint4(a.z, a.w, b.z, b.w);
     }
   };
 
@@ -401,7 +402,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const bf16x8_t va =
-            *reinterpret_cast<const bf16x8_t*>(v_lds + (((pr * NJ + j) * 4 + quad) * 16 + col) * 8);
+            *reinterpret_cast<const bf16x8_t*>(v_lds + (((pr * NJ + j) * 4 + quad) * 16 + (col ^ (8 * (quad >> 1)))) * 8);
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
           o_acc[ct][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[ct][pr], o_acc[ct][j], 0, 0, 0);
@@ -467,12 +468,15 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
   const int bq = (64 * CT) / g;
   // every request may end in a ragged tile and have an odd number of tiles
   const int max_pairs = single ? (T + bq - 1) / bq + R : ((T + bq - 1) / bq + R) / 2 + R;
-  constexpr int lds_bytes = 2 * tile_bytes<D>();
+  // key tiles of 64 (tiles of 32, with which more blocks would fit a compute unit, were slower:
+  // 2,048 tokens 121 against 90 us)
+  constexpr int KB = 4;
+  constexpr int lds_bytes = 2 * tile_bytes<D, KB>();
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&prefill_attention_kernel<D, CT>),
+      reinterpret_cast<const void*>(&prefill_attention_kernel<D, CT, KB>),
       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
   if (attr != hipSuccess) return kvc_fail("kvc_prefill_attention: the kernel's LDS size was refused");
-  hipLaunchKernelGGL((prefill_attention_kernel<D, CT>), dim3(max_pairs, nkv, nsplit), dim3(kWaves * 64),
+  hipLaunchKernelGGL((prefill_attention_kernel<D, CT, KB>), dim3(max_pairs, nkv, nsplit), dim3(kWaves * 64),
                      lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                      q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, part_o,
                      part_ml, single);
