@@ -1,16 +1,16 @@
-// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for 17 to 64 rows of bfloat16, float32 sums: the
-// decode step of a few dozen requests.  The weight matrix is still read once from HBM,
-// but the activations are no longer small beside a wave's share of it, so the waves of a
-// block share them through LDS instead of each reading its own copy from the cache.
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for up to 64 rows of bfloat16 (used from 9 on),
+// float32 sums: the decode step of a few dozen requests.  The weight matrix is still read
+// once from HBM, but the activations are no longer small beside a wave's share of it, so the
+// waves of a block share them through LDS instead of each reading its own copy from the cache.
 //
 // A block of WAVES waves owns WAVES * 16 * RT weight rows and a slice of K.  Each wave
 // walks its 16 * RT rows along the slice in steps of 64, with the weights of the next four
 // to eight steps on their way into registers (a lane loads 16 bytes of one row, a row reads
 // 128 contiguous bytes a step, and the four steps of a chunk are asked for together).  The
 // rows of A of the slice pass through two LDS buffers in chunks of 256 along K, fetched by
-// all waves together as far ahead as the weights: one barrier a chunk.  All loads are issued without a branch around them (addresses beyond the slice
-// are bent back into it and their values never multiplied), so that the waits can count
-// them exactly and none drains the queue.
+// all waves together as far ahead as the weights: one barrier a chunk.  All loads are issued
+// without a branch around them (addresses beyond the slice are bent back into it and their
+// values never multiplied), so that the waits can count them exactly and none drains the queue.
 //
 //   C^T[16 weight rows, 16 tokens] += W[16 rows, 32 k] * A^T[32 k, 16 tokens]   (16x16x32)
 //
