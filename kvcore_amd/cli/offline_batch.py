@@ -44,6 +44,9 @@ def parse_args(argv=None) -> argparse.Namespace:
     p.add_argument("--max-num-partial-prefills", type=int, default=128)
     p.add_argument("--max-long-partial-prefills", type=int, default=128)
     p.add_argument("--long-prefill-token-threshold", type=int, default=0)
+    p.add_argument("--decode-run-ahead", action=argparse.BooleanOptionalAction, default=True,
+                   help="while requests only decode, launch the next step before the tokens of the "
+                        "step in flight have reached the host")
     p.add_argument("--num-gpu-blocks", type=int, default=None)
     p.add_argument("--gpu-memory-utilization", type=float, default=0.9)
     p.add_argument("--random-weights", action="store_true",
@@ -114,6 +117,7 @@ def build_config(args: argparse.Namespace):
             max_num_partial_prefills=args.max_num_partial_prefills,
             max_long_partial_prefills=args.max_long_partial_prefills,
             long_prefill_token_threshold=args.long_prefill_token_threshold,
+            decode_run_ahead=args.decode_run_ahead,
         ),
         device_config=DeviceConfig(device=args.device),
     )

@@ -93,13 +93,16 @@ class CacheConfig:
 
 @dataclass(frozen=True)
 class SchedulerConfig:
-    """Reference: config.py:63-93 (same five names, same validation)."""
+    """Reference: config.py:63-93 (same five names, same validation).  ``decode_run_ahead``
+    is this engine's own: while requests only decode, the next step is launched before the
+    tokens of the step in flight have reached the host (``Scheduler.plan_decode_ahead``)."""
 
     max_num_seqs: int = 8
     max_num_scheduled_tokens: int = 512
     max_num_partial_prefills: int = 1
     max_long_partial_prefills: int = 1
     long_prefill_token_threshold: int = 0
+    decode_run_ahead: bool = True
 
     def __post_init__(self) -> None:
         for name in (

@@ -17,7 +17,7 @@ from kvcore_amd.cache.kv_manager import GroupConfig, KVManager, cdiv
 from kvcore_amd.config.engine_config import KVCoreConfig, canonical_dtype
 from kvcore_amd.config.model_config import read_config_json
 from kvcore_amd.sampling.params import SamplingParams
-from kvcore_amd.sampling.sampler import Sampler, SamplingRow
+from kvcore_amd.sampling.sampler import PendingTokens, Sampler, SamplingRow
 
 from .log import get_logger
 from .request import FinishReason, Request
@@ -106,6 +106,8 @@ class EngineCore:
         if self.tokenizer_manager is not None:
             self.stop_token_ids |= self.tokenizer_manager.get_stop_token_ids()
         self._seeds: dict[str, int] = {}
+        self.run_ahead = sched.decode_run_ahead and model.device.type == "cuda"
+        self._in_flight: _Flight | None = None
         self._finished: dict[str, FinishedRequestOutput] = {}
         self.last_step_stats = StepStats()
 
@@ -176,18 +178,29 @@ class EngineCore:
             self._finished[state.request_id] = FinishedRequestOutput(
                 state.request_id, state.output_token_ids, state.finish_reason)
             self._seeds.pop(state.request_id, None)
+        flight, self._in_flight = self._in_flight, None
+        if flight is not None:
+            self._keep_in_flight(flight)
 
     # -------------------------------------------------------------------------- step
     def step(self) -> EngineCoreOutputs:
+        """One model step's results.  While requests only decode, the step after the one
+        whose results are returned is already running (see ``_launch_ahead``)."""
         stats = StepStats()
         t0 = time.perf_counter()
-        out = self.scheduler.schedule()
+        flight = self._in_flight
+        self._in_flight = None
+        if flight is None:
+            out = self.scheduler.schedule()
+            stats.schedule = time.perf_counter() - t0
+            if out.is_empty:
+                self.last_step_stats = stats
+                return EngineCoreOutputs()
+            flight = self._launch(out)
+        out = flight.output
         t1 = time.perf_counter()
-        stats.schedule = t1 - t0
-        if out.is_empty:
-            self.last_step_stats = stats
-            return EngineCoreOutputs()
-        sampled = self.execute(out)
+        ahead = self._launch_ahead(flight) if self.run_ahead else None
+        sampled = dict(zip(flight.row_ids, flight.tokens.result()))
         t2 = time.perf_counter()
         stats.forward_and_sample = t2 - t1
         result = self.scheduler.update_from_outputs(out, sampled, stop_token_ids=self.stop_token_ids)
@@ -195,6 +208,8 @@ class EngineCore:
             self._finished[state.request_id] = FinishedRequestOutput(
                 state.request_id, state.output_token_ids, state.finish_reason)
             self._seeds.pop(state.request_id, None)
+        if ahead is not None:
+            self._keep_in_flight(ahead)
         stats.update = time.perf_counter() - t2
         stats.num_tokens = out.total_num_scheduled_tokens
         stats.num_reqs = len(out.scheduled)
@@ -206,6 +221,11 @@ class EngineCore:
 
     def execute(self, out: SchedulerOutput) -> dict[str, int]:
         """Run one scheduled step and sample where a request's known tokens end."""
+        flight = self._launch(out)
+        return dict(zip(flight.row_ids, flight.tokens.result()))
+
+    def _launch(self, out: SchedulerOutput, device_tokens: torch.Tensor | None = None) -> "_Flight":
+        """Launch a scheduled step and its sampling; wait for nothing."""
         entries = []
         rows: list[SamplingRow] = []
         row_ids: list[str] = []
@@ -218,8 +238,41 @@ class EngineCore:
             if s.samples:
                 rows.append(SamplingRow(s.sampling_params, self._seeds[s.request_id], s.num_output_tokens))
                 row_ids.append(s.request_id)
-        step_out = self.runner.step(entries)
-        if not rows:
-            return {}
-        tokens = self.sampler.sample(step_out.logits, rows)
-        return dict(zip(row_ids, tokens))
+        step_out = self.runner.step(entries, device_tokens)
+        tokens = self.sampler.launch(step_out.logits, rows) if rows else PendingTokens(None, 0)
+        return _Flight(out, row_ids, tokens)
+
+    def _launch_ahead(self, flight: "_Flight") -> "_Flight | None":
+        """Before the tokens of the step in flight are awaited: if the scheduler can say what
+        the next step is without them (requests that only decode), launch it behind the one
+        in flight, each request's token being read from where that one's sampling leaves it.
+        The host's work for a step then overlaps the device's work for the step before.  A
+        request that turns out to have ended on a stop token has run one token too many,
+        which is dropped (``_keep_in_flight``); its keys and values went to pages that
+        were still its own."""
+        if flight.row_ids != [s.request_id for s in flight.output.scheduled]:
+            return None  # a request was dropped from it: its rows are not the next step's rows
+        planned = self.scheduler.plan_decode_ahead(flight.output)
+        if planned is None:
+            return None
+        return self._launch(planned, flight.tokens.device)
+
+    def _keep_in_flight(self, flight: "_Flight") -> None:
+        """The step launched ahead becomes the step in flight, without the requests that
+        have ended meanwhile."""
+        out = self.scheduler.without_finished(flight.output)
+        if out.is_empty:
+            return
+        if out is not flight.output:
+            flight = _Flight(out, flight.row_ids, flight.tokens)
+        self._in_flight = flight
+
+
+@dataclass
+class _Flight:
+    """A launched step: what was scheduled, the requests of the sampled rows in row order
+    (all of them, also those dropped from ``output`` since) and the tokens on their way."""
+
+    output: SchedulerOutput
+    row_ids: list[str]
+    tokens: PendingTokens

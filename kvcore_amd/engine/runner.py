@@ -220,11 +220,16 @@ class ModelRunner:
         return out
 
     # --------------------------------------------------------------------------- step
-    def step(self, entries: Sequence[StepEntry]) -> StepOutput:
+    def step(self, entries: Sequence[StepEntry], device_tokens: torch.Tensor | None = None) -> StepOutput:
         """Run exactly the tokens given, as one batch, from the cache earlier steps left.
         Keys and values of these tokens are written to their pages first and read back
         from there, so what a position computes does not depend on how its request was
-        cut into steps."""
+        cut into steps.
+
+        ``device_tokens`` (int32 on the device, a value per entry) stands for the token ids
+        of a step of single tokens whose values the host does not know yet: entry ``i``
+        runs ``device_tokens[i]`` as of the time the stream gets here, and the ids in the
+        entries are ignored."""
         R = len(entries)
         if R == 0:
             return StepOutput([], None)
@@ -242,10 +247,16 @@ class ModelRunner:
             self._copy_done.synchronize()
             self._copy_pending = False
         decode_only = all(len(e.tokens) == 1 for e in entries)
+        if device_tokens is not None:
+            if not decode_only:
+                raise ValueError("tokens held by the device stand for single tokens only")
+            if (device_tokens.dtype != torch.int32 or device_tokens.device != self.device
+                    or device_tokens.numel() < R):
+                raise ValueError(f"device_tokens must hold {R} int32 values on {self.device}")
         if decode_only:
             # single tokens only: the same checks and arrays as below, without a loop of
             # array operations per request
-            toks = [e.tokens[0] for e in entries]
+            toks = [0] * R if device_tokens is not None else [e.tokens[0] for e in entries]
             starts = [e.start for e in entries]
             slot_list = [e.slot for e in entries]
             if min(toks) < 0 or max(toks) >= vocab:
@@ -348,6 +359,8 @@ class ModelRunner:
         self._meta_dev[:cursor].copy_(self._meta_host[:cursor], non_blocking=True)
         self._copy_done.record()
         self._copy_pending = True
+        if device_tokens is not None:
+            self._dev["token_ids"][:R].copy_(device_tokens[:R])
         for g, (off, count) in enumerate(upd_counts):
             if count:
                 ops.table_update(self.groups[g].table, self._meta_dev[off:off + 3 * count], count)

@@ -30,6 +30,8 @@ from kvcore_amd.sampling.params import SamplingParams
 
 from .request import FinishReason, Request, RequestStatus
 
+AHEAD_TOKEN = -1  # stands for a token that the device holds and the host does not know yet
+
 
 @dataclass(frozen=True)
 class ScheduledRequest:
@@ -272,6 +274,56 @@ class Scheduler:
             return SchedulerOutput(step_id=self.step_id)
         return SchedulerOutput(tuple(scheduled), num_scheduled, total, finished, tuple(preempted),
                                self.step_id)
+
+    # --------------------------------------------------------------------- run ahead
+    def plan_decode_ahead(self, output: SchedulerOutput) -> SchedulerOutput | None:
+        """The step that follows ``output`` if no request of ``output`` ends on a stop token,
+        made before ``output``'s sampled tokens are known: the same requests in the same
+        order, one position further, the token itself being ``AHEAD_TOKEN`` (the caller
+        takes it from where the device left the sampled one).  Only a step of single
+        decoded tokens that holds every running request is continued, and only if nothing
+        waits, no request reaches its length cap or the context limit with ``output``, no
+        cache group has a window, and every page the next position needs is free: in every
+        other case the answer is None and the caller goes the ordinary way (``update`` then
+        ``schedule``), which decides what this method does not.  Pages are taken at once;
+        a request that ends after all gives them back with the rest of its pages.  The
+        requests themselves are not touched: ``update_from_outputs`` takes the planned step
+        as it takes any other, once it has taken ``output``."""
+        if not output.scheduled or output.preempted_req_ids or self.waiting:
+            return None
+        if len(output.scheduled) != len(self.running):
+            return None
+        if any(g.window > 0 for g in self.kv_manager.groups):
+            return None
+        for s, request in zip(output.scheduled, self.running):
+            if s.request_id != request.request_id or len(s.token_ids) != 1 or not s.samples or s.is_new:
+                return None
+            if s.num_output_tokens + 1 >= request.max_tokens:
+                return None  # ends with ``output``
+            if s.num_computed_tokens + 2 > self.max_model_len:
+                return None
+        planned: list[ScheduledRequest] = []
+        for s in output.scheduled:
+            start = s.num_computed_tokens + 1
+            if self.kv_manager.allocate(s.request_id, start, 1) is None:
+                return None  # pages already taken for others are theirs one step early
+            planned.append(ScheduledRequest(
+                request_id=s.request_id, slot=s.slot, is_new=False, token_ids=(AHEAD_TOKEN,),
+                num_computed_tokens=start,
+                page_ids=tuple(tuple(p) for p in self.kv_manager.page_ids(s.request_id)),
+                released=s.released, samples=True, num_output_tokens=s.num_output_tokens + 1,
+                sampling_params=s.sampling_params))
+        return SchedulerOutput(tuple(planned), {s.request_id: 1 for s in planned}, len(planned),
+                               frozenset(), (), output.step_id + 1)
+
+    def without_finished(self, output: SchedulerOutput) -> SchedulerOutput:
+        """``output`` without the requests that have ended since it was planned."""
+        alive = tuple(s for s in output.scheduled if s.request_id in self.requests)
+        if len(alive) == len(output.scheduled):
+            return output
+        return SchedulerOutput(alive, {s.request_id: len(s.token_ids) for s in alive},
+                               sum(len(s.token_ids) for s in alive), output.finished_req_ids,
+                               output.preempted_req_ids, output.step_id)
 
     # ------------------------------------------------------------------------- update
     def update_from_outputs(self, output: SchedulerOutput, sampled_token_ids: Mapping[str, int], *,

@@ -29,7 +29,8 @@ def folders(tmp_path_factory):
     return out
 
 
-def make_engine(folder, dtype, page, *, num_pages=None, max_seqs=4, budget=64, partial=4, threshold=0):
+def make_engine(folder, dtype, page, *, num_pages=None, max_seqs=4, budget=64, partial=4, threshold=0,
+                run_ahead=True):
     from kvcore_amd import (CacheConfig, KVCoreConfig, LoadConfig, ModelConfig, SchedulerConfig)
     from kvcore_amd.engine.llm_engine import LLMEngine
 
@@ -39,7 +40,8 @@ def make_engine(folder, dtype, page, *, num_pages=None, max_seqs=4, budget=64, p
         cache_config=CacheConfig(block_size=page, num_gpu_blocks=num_pages),
         scheduler_config=SchedulerConfig(max_num_seqs=max_seqs, max_num_scheduled_tokens=budget,
                                          max_num_partial_prefills=partial, max_long_partial_prefills=partial,
-                                         long_prefill_token_threshold=threshold),
+                                         long_prefill_token_threshold=threshold,
+                                         decode_run_ahead=run_ahead),
     ))
 
 
@@ -128,6 +130,52 @@ def test_generation_survives_running_out_of_pages(folders):
     tiny = make_engine(folder, "float32", page, num_pages=4)  # 3 usable pages hold 48 tokens
     with pytest.raises(ValueError, match="cache pages"):
         tiny.add_request("big", SamplingParams(max_tokens=10), prompt_token_ids=list(range(50)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("temperature", [0.0, 0.9])
+def test_steps_launched_ahead_give_the_tokens_of_steps_taken_one_by_one(folders, dtype, temperature):
+    """While requests only decode, the engine launches the next step before it has seen the
+    tokens of the step in flight.  Requests that stop on a token (and so have run one step
+    too far), that reach their length cap and that arrive later must come out as they do
+    from an engine that takes every step by itself."""
+    from kvcore_amd import SamplingParams
+
+    folder, cfg, weights, page = folders["A"]
+    prompts = {f"r{i}": random_tokens(n, 256, seed=500 + i) for i, n in enumerate((9, 17, 30, 5, 12))}
+    caps = {"r0": 40, "r1": 23, "r2": 40, "r3": 31, "r4": 12}
+
+    def run(run_ahead, stop):
+        engine = make_engine(folder, dtype, page, run_ahead=run_ahead, max_seqs=4)
+        engine.engine_core.stop_token_ids = set(stop)
+        launched = 0
+        core = engine.engine_core
+        for i, (rid, p) in enumerate(prompts.items()):
+            if i == 4:
+                continue
+            core.add_request(rid, SamplingParams(max_tokens=caps[rid], temperature=temperature, seed=40 + i),
+                             prompt_token_ids=p)
+        steps = 0
+        while core.has_unfinished_requests():
+            core.step()
+            steps += 1
+            launched += core._in_flight is not None
+            if steps == 6:  # a late arrival, while the others decode
+                core.add_request("r4", SamplingParams(max_tokens=caps["r4"], temperature=temperature, seed=44),
+                                 prompt_token_ids=prompts["r4"])
+        outs = {rid: core.take_finished_output(rid) for rid in prompts}
+        assert core.kv_manager.num_free_pages() == [core.num_pages - 1]
+        assert core.kv_manager.slots.num_free == 4
+        return {rid: (o.output_token_ids, o.finish_reason) for rid, o in outs.items()}, launched
+
+    free, _ = run(False, ())
+    # stop on tokens that r0 and r2 say in mid-course
+    stop = {free["r0"][0][14], free["r2"][0][20]}
+    want, none_ahead = run(False, stop)
+    got, ahead = run(True, stop)
+    assert none_ahead == 0 and ahead > 10
+    assert any(reason.value == "stop" for _, reason in want.values())
+    assert got == want
 
 
 def test_stop_token_ends_a_request(folders):

@@ -232,3 +232,134 @@ def test_random_traffic_keeps_the_invariants(seed):
     assert {k: len(v.output_token_ids) for k, v in finished.items()} == expected
     assert s.kv_manager.num_free_pages() == [s.kv_manager.pools[0].num_usable]
     assert s.kv_manager.slots.num_free == 4
+
+
+# ------------------------------------------------------------------------ running ahead
+def _fake_token(rid, index, stop_at):
+    """A request's ``index``-th output: a function of the request and the index alone, as the
+    engine's tokens are; request ``rid`` says the stop token 99 at index ``stop_at[rid]``."""
+    return 99 if stop_at.get(rid) == index else 100 + (hash((rid, index)) % 50)
+
+
+def _drive(scheduler, *, ahead, stop_at, arrivals=()):
+    """The engine's loop without a device: with ``ahead`` the step after the one whose tokens
+    are awaited is planned first, as ``EngineCore.step`` does.  Returns each request's output
+    and the requests of every step that ran."""
+    outputs, steps = {}, []
+    stats = {"planned": 0, "dropped": 0}
+    arrivals = dict(arrivals)
+    in_flight = None
+    for tick in range(400):
+        for request in arrivals.pop(tick, ()):
+            scheduler.add_request(request)
+        if not scheduler.has_unfinished_requests():
+            if not arrivals:
+                break
+            continue
+        out, in_flight = in_flight, None
+        if out is None:
+            out = scheduler.schedule()
+            if out.is_empty:
+                continue
+        steps.append(tuple((s.request_id, s.num_computed_tokens, len(s.token_ids)) for s in out.scheduled))
+        planned = scheduler.plan_decode_ahead(out) if ahead else None
+        sampled = {s.request_id: _fake_token(s.request_id, s.num_output_tokens, stop_at)
+                   for s in out.scheduled if s.samples}
+        result = scheduler.update_from_outputs(out, sampled, stop_token_ids={99})
+        for state in result.finished_requests:
+            outputs[state.request_id] = (state.output_token_ids, state.finish_reason)
+        if planned is not None:
+            stats["planned"] += 1
+            kept = scheduler.without_finished(planned)
+            stats["dropped"] += len(planned.scheduled) - len(kept.scheduled)
+            in_flight = None if kept.is_empty else kept
+    assert not scheduler.has_unfinished_requests()
+    return outputs, steps, stats
+
+
+def test_a_step_planned_ahead_is_the_step_that_would_have_been_scheduled():
+    s = make_scheduler(SchedulerConfig(max_num_seqs=4, max_num_scheduled_tokens=16, max_num_partial_prefills=4),
+                       num_pages=32, page=2, max_len=24)
+    s.add_request(make_request("a", [1, 2, 3], max_tokens=6))
+    s.add_request(make_request("b", [4, 5, 6, 7], max_tokens=6))
+    first = s.schedule()
+    assert s.plan_decode_ahead(first) is None  # prompts: not a step of single decoded tokens
+    s.update_from_outputs(first, {"a": 10, "b": 11})
+    second = s.schedule()
+    planned = s.plan_decode_ahead(second)
+    assert planned is not None and planned.step_id == second.step_id + 1
+    s.update_from_outputs(second, {"a": 12, "b": 13})
+    # what the ordinary way would schedule now, the tokens aside, is what was planned
+    pages = {r.request_id: s.kv_manager.page_ids(r.request_id) for r in s.running}
+    for share, request in zip(planned.scheduled, s.running):
+        assert share.request_id == request.request_id
+        assert share.num_computed_tokens == request.num_computed_tokens
+        assert share.token_ids == (-1,) and share.samples and not share.is_new
+        assert share.num_output_tokens == request.num_output_tokens
+        assert [list(p) for p in share.page_ids] == [list(p) for p in pages[request.request_id]]
+        assert len(share.page_ids[0]) * 2 > share.num_computed_tokens
+    s.update_from_outputs(planned, {"a": 14, "b": 15})
+    assert s.requests["a"].output_token_ids[-3:] == [10, 12, 14]
+
+
+def test_nothing_is_planned_ahead_when_the_ordinary_way_has_something_to_decide():
+    config = SchedulerConfig(max_num_seqs=4, max_num_scheduled_tokens=16, max_num_partial_prefills=4)
+    # a request reaches its length cap with the step
+    s = make_scheduler(config, num_pages=32, max_len=24)
+    s.add_request(make_request("a", [1, 2, 3], max_tokens=2))
+    s.update_from_outputs(s.schedule(), {"a": 10})
+    assert s.plan_decode_ahead(s.schedule()) is None
+    # another request waits
+    s = make_scheduler(config, num_pages=32, max_len=24)
+    s.add_request(make_request("a", [1, 2, 3], max_tokens=8))
+    s.update_from_outputs(s.schedule(), {"a": 10})
+    out = s.schedule()
+    s.add_request(make_request("b", [1], max_tokens=2))
+    assert s.plan_decode_ahead(out) is None
+    # no page is free for the next position
+    s = make_scheduler(config, num_pages=4, page=2, max_len=6)
+    s.add_request(make_request("a", [1, 2, 3], max_tokens=3))
+    s.add_request(make_request("b", [4], max_tokens=2))
+    s.update_from_outputs(s.schedule(), {"a": 10, "b": 11})
+    out = s.schedule()  # a: position 3 (page 2 of 2), b: position 1; three pages are out
+    assert s.kv_manager.num_free_pages() == [0] and s.plan_decode_ahead(out) is None
+    # a window gives pages back as a request goes
+    s = make_scheduler(config, num_pages=32, max_len=24, window=4)
+    s.add_request(make_request("a", [1, 2, 3], max_tokens=8))
+    s.update_from_outputs(s.schedule(), {"a": 10})
+    assert s.plan_decode_ahead(s.schedule()) is None
+    # the context limit
+    s = make_scheduler(config, num_pages=32, max_len=5)
+    s.add_request(make_request("a", [1, 2, 3], max_tokens=2))
+    s.update_from_outputs(s.schedule(), {"a": 10})
+    assert s.plan_decode_ahead(s.schedule()) is None
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_running_ahead_gives_the_outputs_of_the_ordinary_way(seed):
+    """Stop tokens at random places (a request that stops has been planned one step too far),
+    length caps, arrivals while others decode, and a pool small enough to preempt."""
+    rng = random.Random(seed)
+    specs, stop_at, arrivals = [], {}, {}
+    for i in range(7):
+        rid = f"r{i}"
+        specs.append((rid, [rng.randrange(50) for _ in range(rng.randint(1, 9))], rng.randint(1, 12)))
+        if rng.random() < 0.6:
+            stop_at[rid] = rng.randint(0, 8)
+        arrivals.setdefault(0 if i < 3 else rng.randint(1, 25), []).append(i)
+    results = []
+    for ahead in (False, True):
+        s = make_scheduler(SchedulerConfig(max_num_seqs=4, max_num_scheduled_tokens=8, max_num_partial_prefills=2),
+                           num_pages=rng.choice([14, 40]) if not results else results[0][2], page=2, max_len=24)
+        pool = s.kv_manager.pools[0].num_usable + 1
+        arriving = {t: [make_request(*specs[i]) for i in ids] for t, ids in arrivals.items()}
+        outputs, steps, stats = _drive(s, ahead=ahead, stop_at=stop_at, arrivals=arriving)
+        assert s.kv_manager.num_free_pages() == [s.kv_manager.pools[0].num_usable]
+        results.append((outputs, steps, pool, stats))
+    assert results[0][0] == results[1][0]
+    assert results[1][3]["planned"] > 0
+    print("planned ahead", results[1][3], "of", len(results[1][1]), "steps")
+    assert set(results[0][0]) == {rid for rid, _, _ in specs}
+    for rid, (tokens, reason) in results[1][0].items():
+        if rid in stop_at and stop_at[rid] < len(tokens):
+            assert tokens[-1] == 99 and reason == FinishReason.STOP
