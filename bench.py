@@ -62,7 +62,8 @@ def parse_args():
     p.add_argument("--model", default="8b", choices=sorted(MODELS),
                    help="layer sizes: 8b is the headline configuration; 1b and 70b are the other "
                         "shapes of the baseline")
-    p.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="prompt length of the decode runs")
+    p.add_argument("--prompt-len", type=int, default=None,
+                   help="prompt length of the decode runs (default 512; 1,024 for the 70b shape)")
     p.add_argument("--mixed", action="store_true",
                    help="instead of the decode runs: 64 requests with prompts of 16..2048 tokens, "
                         "portions of 512, 128 new tokens each, timed as a whole")
@@ -110,7 +111,7 @@ def main() -> int:
 
     model_name, base_cfg = MODELS[args.model]
     cfg = dict(base_cfg)
-    prompt_len = args.prompt_len
+    prompt_len = args.prompt_len or (1024 if args.model == "70b" else PROMPT_LEN)
     full_layers = cfg["num_hidden_layers"]
     if args.layers is not None:
         cfg["num_hidden_layers"] = args.layers
