@@ -282,15 +282,17 @@ class Scheduler:
         order, one position further, the token itself being ``AHEAD_TOKEN`` (the caller
         takes it from where the device left the sampled one).  Only a step of single
         decoded tokens that holds every running request is continued, and only if nothing
-        waits, no request reaches its length cap or the context limit with ``output``, no
+        waits that a free slot could take, no request reaches its length cap or the context limit with ``output``, no
         cache group has a window, and every page the next position needs is free: in every
         other case the answer is None and the caller goes the ordinary way (``update`` then
         ``schedule``), which decides what this method does not.  Pages are taken at once;
         a request that ends after all gives them back with the rest of its pages.  The
         requests themselves are not touched: ``update_from_outputs`` takes the planned step
         as it takes any other, once it has taken ``output``."""
-        if not output.scheduled or output.preempted_req_ids or self.waiting:
+        if not output.scheduled or output.preempted_req_ids:
             return None
+        if self.waiting and self.kv_manager.has_free_slot():
+            return None  # with every slot taken nobody can be admitted (``schedule``, pass 2)
         if len(output.scheduled) != len(self.running):
             return None
         if any(g.window > 0 for g in self.kv_manager.groups):

@@ -178,6 +178,39 @@ def test_steps_launched_ahead_give_the_tokens_of_steps_taken_one_by_one(folders,
     assert got == want
 
 
+def test_abort_while_a_step_is_in_flight(folders):
+    """A request aborted while the step launched ahead still holds it: the step's row for it
+    is dropped, the others go on as if nothing had happened."""
+    from kvcore_amd import SamplingParams
+
+    folder, cfg, weights, page = folders["A"]
+    prompts = {f"r{i}": random_tokens(n, 256, seed=700 + i) for i, n in enumerate((11, 6, 21))}
+
+    def run(abort_at):
+        core = make_engine(folder, "float32", page).engine_core
+        for rid, p in prompts.items():
+            core.add_request(rid, SamplingParams(max_tokens=20, temperature=0.0, ignore_eos=True),
+                             prompt_token_ids=p)
+        steps = 0
+        while core.has_unfinished_requests():
+            core.step()
+            steps += 1
+            if steps == abort_at:
+                assert core._in_flight is not None
+                core.abort_requests(["r1"])
+                assert all(s.request_id != "r1" for s in core._in_flight.output.scheduled)
+        assert core.kv_manager.num_free_pages() == [core.num_pages - 1]
+        return {rid: core.take_finished_output(rid) for rid in prompts}
+
+    whole = run(None)
+    cut = run(5)
+    assert cut["r1"].finish_reason.value == "abort"
+    assert cut["r1"].output_token_ids == whole["r1"].output_token_ids[:len(cut["r1"].output_token_ids)]
+    assert 0 < len(cut["r1"].output_token_ids) < 20
+    for rid in ("r0", "r2"):
+        assert cut[rid].output_token_ids == whole[rid].output_token_ids and len(cut[rid].output_token_ids) == 20
+
+
 def test_stop_token_ends_a_request(folders):
     from kvcore_amd import SamplingParams
 

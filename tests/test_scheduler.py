@@ -309,13 +309,21 @@ def test_nothing_is_planned_ahead_when_the_ordinary_way_has_something_to_decide(
     s.add_request(make_request("a", [1, 2, 3], max_tokens=2))
     s.update_from_outputs(s.schedule(), {"a": 10})
     assert s.plan_decode_ahead(s.schedule()) is None
-    # another request waits
+    # another request waits and a slot is free for it
     s = make_scheduler(config, num_pages=32, max_len=24)
     s.add_request(make_request("a", [1, 2, 3], max_tokens=8))
     s.update_from_outputs(s.schedule(), {"a": 10})
     out = s.schedule()
     s.add_request(make_request("b", [1], max_tokens=2))
     assert s.plan_decode_ahead(out) is None
+    # ... but with every slot taken the waiting request changes nothing
+    one = SchedulerConfig(max_num_seqs=1, max_num_scheduled_tokens=16)
+    s = make_scheduler(one, num_pages=32, max_len=24)
+    s.add_request(make_request("a", [1, 2, 3], max_tokens=8))
+    s.update_from_outputs(s.schedule(), {"a": 10})
+    out = s.schedule()
+    s.add_request(make_request("b", [1], max_tokens=2))
+    assert s.plan_decode_ahead(out) is not None
     # no page is free for the next position
     s = make_scheduler(config, num_pages=4, page=2, max_len=6)
     s.add_request(make_request("a", [1, 2, 3], max_tokens=3))
