@@ -200,20 +200,39 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     const int rem = (D == 128) ? tid : (tid & 127);
     v_off[i] = (rem >> 1) * page_size + (rem & 1) * 8;
   }
-  auto fetch_tile = [&](int kb0) {
+  // The page ids of a tile are looked up one tile before the tile is fetched: a lookup is a
+  // scalar load whose answer the fetch would otherwise wait for, four times in a row per tile.
+  // The lookups walk the key blocks in order, so page index and block within the page are
+  // counted along instead of divided out.
+  int look_kb = 0, look_page_index = 0, look_sub = 0;
+  auto seek_pages = [&](int kb) {
+    look_kb = kb;
+    look_page_index = kb / blocks_per_page;
+    look_sub = kb - look_page_index * blocks_per_page;
+  };
+  // page id (or -1: none, or not a page) and 16-key block within the page, for the tile at the cursor
+  auto lookup_pages = [&](int (&page)[kKeyBlocks], int (&sub)[kKeyBlocks]) {
+#pragma unroll
+    for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
+      page[kbi] = -1;
+      sub[kbi] = look_sub;
+      if (look_kb < kb_end) page[kbi] = __builtin_amdgcn_readfirstlane(row_table[look_page_index]);
+      ++look_kb;
+      if (++look_sub == blocks_per_page) {
+        look_sub = 0;
+        ++look_page_index;
+      }
+    }
+  };
+  auto fetch_tile = [&](int kb0, const int (&page)[kKeyBlocks], const int (&sub)[kKeyBlocks]) {
     const bool tail = (kb0 + kKeyBlocks) * 16 > pos_hi + 1;  // uniform: some keys are not the request's
     int64_t kpage[kKeyBlocks], vpage[kKeyBlocks];  // element offsets of the key blocks, or -1
 #pragma unroll
     for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
-      const int kb = kb0 + kbi;
       kpage[kbi] = vpage[kbi] = -1;
-      if (kb < kb_end) {
-        const int page = __builtin_amdgcn_readfirstlane(row_table[kb / blocks_per_page]);
-        if (page > 0 && page < num_pages) {
-          const int sub = kb % blocks_per_page;
-          kpage[kbi] = ((static_cast<int64_t>(page) * nkv + hk) * page_size + sub * 16) * D;
-          vpage[kbi] = (static_cast<int64_t>(page) * nkv + hk) * D * page_size + sub * 16;
-        }
+      if (page[kbi] > 0 && page[kbi] < num_pages) {
+        kpage[kbi] = ((static_cast<int64_t>(page[kbi]) * nkv + hk) * page_size + sub[kbi] * 16) * D;
+        vpage[kbi] = (static_cast<int64_t>(page[kbi]) * nkv + hk) * D * page_size + sub[kbi] * 16;
       }
     }
     if (!tail) {
@@ -417,13 +436,20 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   const int kb_mine = kb_first + static_cast<int>(blockIdx.z) * tiles_mine * kKeyBlocks;
   const int kb_mine_end = (kb_mine + tiles_mine * kKeyBlocks < kb_end) ? kb_mine + tiles_mine * kKeyBlocks : kb_end;
   if (kb_mine < kb_mine_end) {  // the same for the whole block
-    fetch_tile(kb_mine);
+    int page[kKeyBlocks], sub[kKeyBlocks];
+    seek_pages(kb_mine);
+    lookup_pages(page, sub);
+    fetch_tile(kb_mine, page, sub);
+    lookup_pages(page, sub);  // of the second tile
     store_tile(0);
     __syncthreads();
     int buf = 0;
     for (int kb0 = kb_mine; kb0 < kb_mine_end; kb0 += kKeyBlocks, buf ^= 1) {
       const bool more = kb0 + kKeyBlocks < kb_mine_end;
-      if (more) fetch_tile(kb0 + kKeyBlocks);  // in flight while this tile is used
+      if (more) {
+        fetch_tile(kb0 + kKeyBlocks, page, sub);  // in flight while this tile is used
+        lookup_pages(page, sub);                  // of the tile after it, answered by then
+      }
       if (kb0 * 16 <= wave_pos_hi) work_tile(kb0, buf);  // scalar: else nothing here is visible to this wave
       if (more) store_tile(buf ^ 1);
       __syncthreads();  // the next tile is whole, and this one has been consumed
