@@ -1,9 +1,10 @@
 // Paged attention for portions of prompts, bfloat16, on the matrix cores.
 //
-// A block of four waves owns up to 64*CT query rows of one request and one kv head:
-// BQ = 64*CT / g consecutive tokens times the g query heads that share the kv head.
-// It walks the request's keys in tiles of 64, staged once through LDS for all four
-// waves (two tiles of LDS: while one is read, the next is written, one barrier a tile):
+// A block of W = 4 or 8 waves owns up to 16*W*CT query rows of one request and one kv head:
+// BQ = 16*W*CT / g consecutive tokens times the g query heads that share the kv head.
+// It walks the request's keys in tiles of 64 (128 for eight waves on heads of 64), staged
+// once through LDS for all its waves (two tiles of LDS: while one is read, the next is
+// written, one barrier a tile):
 // K pages as they lie in the cache ([key, d], rows padded against bank conflicts) and V
 // pages ([d, key]) regrouped so that operand reads are contiguous.  Per wave:
 //
@@ -46,7 +47,6 @@ __device__ __forceinline__ s16x4_t pack_bf16x4(const float* p) {
   return *reinterpret_cast<s16x4_t*>(&v);
 }
 
-constexpr int kWaves = 4;
 
 // KB: 16-key blocks per LDS tile
 template <int D, int KB>
@@ -54,8 +54,10 @@ constexpr int tile_bytes() {
   return KB * 16 * (D + 16) * 2 + KB * D * 16 * 2;  // K rows padded, then V
 }
 
-template <int D, int CT, int KB>
-__global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
+// W: waves of a block (4 or 8).  Eight waves stage each key tile for twice the rows, which
+// halves the block's loads and LDS writes per row; a compute unit then holds one block.
+template <int D, int CT, int KB, int W>
+__global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ table, int table_stride, const int32_t* __restrict__ positions,
@@ -73,8 +75,28 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   extern __shared__ __attribute__((aligned(16))) bf16_t tiles[];  // two tiles: [K | V] each
 
   const int g = nh / nkv;
-  const int bq = (64 * CT) / g;  // tokens per block
-  const int hk = blockIdx.y;
+  const int bq = (16 * W * CT) / g;  // tokens per block
+  // Workgroups go to the chip's eight dies in turn (workgroup id modulo 8) and every die has
+  // an L2 of its own, while all blocks of a kv head read the same keys and values.  So a kv
+  // head's blocks get ids that land on one die (with fewer than eight kv heads, on 8 / nkv
+  // dies): the die's L2 then holds one head's keys and values instead of every head's.
+  // Head counts that neither divide eight nor are divided by it are dealt out plainly.
+  int hk, block_index;
+  {
+    const int lin = blockIdx.x;  // the grid is a multiple of 8 wide
+    const int die = lin & 7, turn = lin >> 3;
+    if ((nkv & 7) == 0) {
+      const int per_die = nkv >> 3;
+      hk = die + 8 * (turn % per_die);
+      block_index = turn / per_die;
+    } else if (8 % nkv == 0) {
+      hk = die % nkv;
+      block_index = turn * (8 / nkv) + die / nkv;
+    } else {
+      hk = lin % nkv;
+      block_index = lin / nkv;
+    }
+  }
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
@@ -87,7 +109,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   // about the same number of key tiles.  Pairs are numbered request by request.
   int req = -1, pair = 0, n_tiles = 0, q_begin = 0, q_end = 0;
   {
-    int idx = blockIdx.x;
+    int idx = block_index;
     for (int r = 0; r < num_reqs; ++r) {
       const int b = q_start[r], e = q_start[r + 1];
       const int tiles_r = (e - b + bq - 1) / bq;
@@ -178,18 +200,32 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   const int kb_end = pos_hi / 16 + 1;
   constexpr int K_CHUNKS = kKeyBlocks * 16 * (D / 8);  // 16-byte pieces of a K tile
   constexpr int V_CHUNKS = kKeyBlocks * D * 2;         // 16-byte pieces of a V tile
-  constexpr int K_PER_THREAD = K_CHUNKS / (kWaves * 64);
-  constexpr int V_PER_THREAD = V_CHUNKS / (kWaves * 64);
+  constexpr int THREADS = W * 64;
+  constexpr int K_PER_THREAD = K_CHUNKS / THREADS;
+  constexpr int V_PER_THREAD = V_CHUNKS / THREADS;
   uint4 kreg[K_PER_THREAD], vreg[V_PER_THREAD];
 
   // Fetch the tile that starts at key block kb0 into registers.  Keys beyond the request's
   // last position, key blocks beyond the range and pages that are gone arrive as zeros.
-  // A thread's pieces of step i all lie in key block i (head size 128) or in key blocks
-  // 2i and 2i+1 (head size 64), so the page lookups are uniform or nearly so.
-  constexpr int PIECES = D / 8;               // 16-byte pieces of a K row
-  constexpr int ROWS_PER_STEP = 256 / PIECES;  // K rows that the block fetches per step
-  const int k_row0 = tid / PIECES;             // this thread's K row within a step
+  // The key blocks that a thread fetches from are the same for its whole wave (K: 16 rows of
+  // 16-byte pieces are 128 or 256 threads; V: a key block takes 2 * D threads), so a wave looks
+  // up the pages of its own key blocks only, as scalars.
+  constexpr int PIECES = D / 8;                    // 16-byte pieces of a K row
+  constexpr int ROWS_PER_STEP = THREADS / PIECES;  // K rows that the block fetches per step
+  // V: a key block's rows of the head times its two halves of 8 keys take V_THREADS threads;
+  // the block's threads form V_GROUPS such groups, each with an even number of key blocks
+  constexpr int V_THREADS = 2 * D;
+  constexpr int V_GROUPS = THREADS / V_THREADS;
+  static_assert(THREADS % V_THREADS == 0 && kKeyBlocks % (2 * V_GROUPS) == 0 &&
+                    V_PER_THREAD == kKeyBlocks / V_GROUPS && (kKeyBlocks * 16) % ROWS_PER_STEP == 0 &&
+                    V_THREADS % 64 == 0 && (16 * PIECES) % 64 == 0,
+                "tile shape and block size do not fit");
+  const int v_group = (V_GROUPS == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid / V_THREADS);  // key blocks v_group * V_PER_THREAD ...
+  const int v_rem = tid % V_THREADS;                                    // (row of the head) * 2 + half
+  const int k_row0 = tid / PIECES;  // this thread's K row within a step
   const int k_piece = tid % PIECES;
+  // the key block within a step's rows that this wave fetches K from (steps of more than 16 rows)
+  const int k_block0 = (ROWS_PER_STEP <= 16) ? 0 : __builtin_amdgcn_readfirstlane(k_row0 >> 4);
   // element offsets of this thread's pieces within a key block's K rows and V rows
   int k_off[K_PER_THREAD], v_off[V_PER_THREAD];
 #pragma unroll
@@ -197,100 +233,83 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     k_off[i] = ((i * ROWS_PER_STEP + k_row0) & 15) * D + k_piece * 8;
 #pragma unroll
   for (int i = 0; i < V_PER_THREAD; ++i) {
-    const int rem = (D == 128) ? tid : (tid & 127);
-    v_off[i] = (rem >> 1) * page_size + (rem & 1) * 8;
+    v_off[i] = (v_rem >> 1) * page_size + (v_rem & 1) * 8;
   }
-  // The page ids of a tile are looked up one tile before the tile is fetched: a lookup is a
-  // scalar load whose answer the fetch would otherwise wait for, four times in a row per tile.
-  // The lookups walk the key blocks in order, so page index and block within the page are
-  // counted along instead of divided out.
-  int look_kb = 0, look_page_index = 0, look_sub = 0;
-  auto seek_pages = [&](int kb) {
-    look_kb = kb;
-    look_page_index = kb / blocks_per_page;
-    look_sub = kb - look_page_index * blocks_per_page;
-  };
-  // page id (or -1: none, or not a page) and 16-key block within the page, for the tile at the cursor
-  auto lookup_pages = [&](int (&page)[kKeyBlocks], int (&sub)[kKeyBlocks]) {
-#pragma unroll
-    for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
-      page[kbi] = -1;
-      sub[kbi] = look_sub;
-      if (look_kb < kb_end) page[kbi] = __builtin_amdgcn_readfirstlane(row_table[look_page_index]);
-      ++look_kb;
-      if (++look_sub == blocks_per_page) {
-        look_sub = 0;
-        ++look_page_index;
+  // Element offsets of this wave's key blocks of the tile at kb0 in the K and V planes, or -1
+  // (no such block, or not a page).  They are looked up one tile before the tile is fetched (a
+  // lookup is a scalar load whose answer the fetch would otherwise wait for) and with as little
+  // scalar arithmetic as possible, which this kernel has much of: a shift where a page holds a
+  // power of two of key blocks, and one 64-bit product per block for both planes.
+  const int sub_mask = blocks_per_page - 1;
+  const int sub_shift = (blocks_per_page & sub_mask) == 0 ? __builtin_ctz(blocks_per_page) : -1;
+  const int64_t page_elems = static_cast<int64_t>(nkv) * page_size * D;  // of one plane
+  const int64_t head_elems = static_cast<int64_t>(hk) * page_size * D;
+  auto block_at = [&](int kb, int64_t& k_at, int64_t& v_at) {
+    k_at = v_at = -1;
+    if (kb < kb_end) {
+      int page_index, sub;
+      if (sub_shift >= 0) {
+        page_index = kb >> sub_shift;
+        sub = kb & sub_mask;
+      } else {
+        page_index = kb / blocks_per_page;
+        sub = kb - page_index * blocks_per_page;
+      }
+      const int page = __builtin_amdgcn_readfirstlane(row_table[page_index]);
+      if (page > 0 && page < num_pages) {
+        const int64_t at = page * page_elems + head_elems;
+        k_at = at + sub * (16 * D);
+        v_at = at + sub * 16;
       }
     }
   };
-  auto fetch_tile = [&](int kb0, const int (&page)[kKeyBlocks], const int (&sub)[kKeyBlocks]) {
+  // whether step i of the K fetch and piece i of the V fetch lie in the same key block for all i
+  constexpr bool kSameBlocks = ROWS_PER_STEP == 16 && V_GROUPS == 1;
+  auto lookup_pages = [&](int kb0, int64_t (&kbase)[K_PER_THREAD], int64_t (&vbase)[V_PER_THREAD]) {
+    if constexpr (kSameBlocks) {
+      static_assert(K_PER_THREAD == V_PER_THREAD, "one key block per step and piece");
+#pragma unroll
+      for (int i = 0; i < K_PER_THREAD; ++i) block_at(kb0 + i, kbase[i], vbase[i]);
+    } else {
+      int64_t unused;
+#pragma unroll
+      for (int i = 0; i < K_PER_THREAD; ++i)
+        block_at(kb0 + (i * ROWS_PER_STEP) / 16 + k_block0, kbase[i], unused);
+#pragma unroll
+      for (int i = 0; i < V_PER_THREAD; ++i) block_at(kb0 + v_group * V_PER_THREAD + i, unused, vbase[i]);
+    }
+  };
+  auto fetch_tile = [&](int kb0, const int64_t (&kbase)[K_PER_THREAD], const int64_t (&vbase)[V_PER_THREAD]) {
     const bool tail = (kb0 + kKeyBlocks) * 16 > pos_hi + 1;  // uniform: some keys are not the request's
-    int64_t kpage[kKeyBlocks], vpage[kKeyBlocks];  // element offsets of the key blocks, or -1
-#pragma unroll
-    for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
-      kpage[kbi] = vpage[kbi] = -1;
-      if (page[kbi] > 0 && page[kbi] < num_pages) {
-        kpage[kbi] = ((static_cast<int64_t>(page[kbi]) * nkv + hk) * page_size + sub[kbi] * 16) * D;
-        vpage[kbi] = (static_cast<int64_t>(page[kbi]) * nkv + hk) * D * page_size + sub[kbi] * 16;
-      }
-    }
     if (!tail) {
       // every key of the tile is the request's: a scalar base and a fixed offset per piece
 #pragma unroll
-      for (int i = 0; i < K_PER_THREAD; ++i) {
-        int64_t base;
-        if constexpr (ROWS_PER_STEP == 16) {
-          base = kpage[i];
-        } else {
-          base = (k_row0 < 16) ? kpage[2 * i] : kpage[2 * i + 1];
-        }
-        kreg[i] = (base >= 0) ? *reinterpret_cast<const uint4*>(k_cache + base + k_off[i])
-                              : make_uint4(0u, 0u, 0u, 0u);
-      }
+      for (int i = 0; i < K_PER_THREAD; ++i)
+        kreg[i] = (kbase[i] >= 0) ? *reinterpret_cast<const uint4*>(k_cache + kbase[i] + k_off[i])
+                                  : make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
-      for (int i = 0; i < V_PER_THREAD; ++i) {
-        int64_t base;
-        if constexpr (D == 128) {
-          base = vpage[i];
-        } else {
-          base = (tid < 128) ? vpage[i] : vpage[2 + i];
-        }
-        vreg[i] = (base >= 0) ? *reinterpret_cast<const uint4*>(v_cache + base + v_off[i])
-                              : make_uint4(0u, 0u, 0u, 0u);
-      }
+      for (int i = 0; i < V_PER_THREAD; ++i)
+        vreg[i] = (vbase[i] >= 0) ? *reinterpret_cast<const uint4*>(v_cache + vbase[i] + v_off[i])
+                                  : make_uint4(0u, 0u, 0u, 0u);
       return;
     }
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
-      const int key_row = i * ROWS_PER_STEP + k_row0;  // 0 .. 63 within the tile
-      int64_t base;
-      if constexpr (ROWS_PER_STEP == 16) {
-        base = kpage[i];
-      } else {
-        static_assert(ROWS_PER_STEP == 32, "head size 64 or 128");
-        base = (k_row0 < 16) ? kpage[2 * i] : kpage[2 * i + 1];
-      }
+      const int key_row = i * ROWS_PER_STEP + k_row0;  // within the tile
       uint4 val = make_uint4(0u, 0u, 0u, 0u);
-      if (base >= 0 && kb0 * 16 + key_row <= pos_hi)
-        val = *reinterpret_cast<const uint4*>(k_cache + base + k_off[i]);
+      if (kbase[i] >= 0 && kb0 * 16 + key_row <= pos_hi)
+        val = *reinterpret_cast<const uint4*>(k_cache + kbase[i] + k_off[i]);
       kreg[i] = val;
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
       // this thread's pieces: both key blocks of a pair, one row of the head, one half of 16 keys
-      const int kbi = (D == 128) ? i : 2 * (tid >> 7) + i;
-      const int half = tid & 1;
-      int64_t base;
-      if constexpr (D == 128) {
-        base = vpage[i];
-      } else {
-        base = (tid < 128) ? vpage[i] : vpage[2 + i];
-      }
+      const int kbi = v_group * V_PER_THREAD + i;
+      const int half = v_rem & 1;
       uint4 val = make_uint4(0u, 0u, 0u, 0u);
       const int key0 = (kb0 + kbi) * 16 + half * 8;
-      if (base >= 0 && key0 <= pos_hi) {
-        val = *reinterpret_cast<const uint4*>(v_cache + base + v_off[i]);
+      if (vbase[i] >= 0 && key0 <= pos_hi) {
+        val = *reinterpret_cast<const uint4*>(v_cache + vbase[i] + v_off[i]);
         const int n_ok = pos_hi - key0 + 1;  // keys key0 .. key0+7 beyond pos_hi are not this request's
         if (n_ok < 8) {
           uint32_t w[4] = {val.x, val.y, val.z, val.w};
@@ -320,10 +339,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
     // 16 different slots; the reads flip it back.
 #pragma unroll
     for (int pr = 0; pr < V_PER_THREAD / 2; ++pr) {
-      const int rem = (D == 128) ? tid : (tid & 127);
-      const int pair = (D == 128) ? pr : (tid >> 7);
-      const int drow = rem >> 1;
-      const int half = rem & 1;
+      const int pair = v_group * (V_PER_THREAD / 2) + pr;
+      const int drow = v_rem >> 1;
+      const int half = v_rem & 1;
       const uint4 a = vreg[2 * pr], b = vreg[2 * pr + 1];
       bf16_t* dst = v_lds + (((pair * NJ + (drow >> 4)) * 4 + 2 * half) * 16 + ((drow & 15) ^ (8 * half))) * 8;
       *reinterpret_cast<uint4*>(dst) = make_uint4(a.x, a.y, b.x, b.y);
@@ -436,19 +454,18 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   const int kb_mine = kb_first + static_cast<int>(blockIdx.z) * tiles_mine * kKeyBlocks;
   const int kb_mine_end = (kb_mine + tiles_mine * kKeyBlocks < kb_end) ? kb_mine + tiles_mine * kKeyBlocks : kb_end;
   if (kb_mine < kb_mine_end) {  // the same for the whole block
-    int page[kKeyBlocks], sub[kKeyBlocks];
-    seek_pages(kb_mine);
-    lookup_pages(page, sub);
-    fetch_tile(kb_mine, page, sub);
-    lookup_pages(page, sub);  // of the second tile
+    int64_t kbase[K_PER_THREAD], vbase[V_PER_THREAD];
+    lookup_pages(kb_mine, kbase, vbase);
+    fetch_tile(kb_mine, kbase, vbase);
+    lookup_pages(kb_mine + kKeyBlocks, kbase, vbase);
     store_tile(0);
     __syncthreads();
     int buf = 0;
     for (int kb0 = kb_mine; kb0 < kb_mine_end; kb0 += kKeyBlocks, buf ^= 1) {
       const bool more = kb0 + kKeyBlocks < kb_mine_end;
       if (more) {
-        fetch_tile(kb0 + kKeyBlocks, page, sub);  // in flight while this tile is used
-        lookup_pages(page, sub);                  // of the tile after it, answered by then
+        fetch_tile(kb0 + kKeyBlocks, kbase, vbase);        // in flight while this tile is used
+        lookup_pages(kb0 + 2 * kKeyBlocks, kbase, vbase);  // answered by the time it is fetched
       }
       if (kb0 * 16 <= wave_pos_hi) work_tile(kb0, buf);  // scalar: else nothing here is visible to this wave
       if (more) store_tile(buf ^ 1);
@@ -484,25 +501,31 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(
   }  // turn
 }
 
-template <int D, int CT>
+template <int D, int CT, int W>
 int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t* k_cache,
                       const bf16_t* v_cache, const int32_t* table, int table_stride,
                       const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                       int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
                       float* part_o, float* part_ml, int nsplit, int single, hipStream_t stream) {
   const int g = nh / nkv;
-  const int bq = (64 * CT) / g;
+  const int bq = (16 * W * CT) / g;
   // every request may end in a ragged tile and have an odd number of tiles
   const int max_pairs = single ? (T + bq - 1) / bq + R : ((T + bq - 1) / bq + R) / 2 + R;
   // key tiles of 64 (tiles of 32, with which more blocks would fit a compute unit, were slower:
   // 2,048 tokens 121 against 90 us)
-  constexpr int KB = 4;
+  // (eight waves on heads of 64 take tiles of 128 keys, so that a thread still stages whole
+  // pairs of key blocks)
+  constexpr int KB = (D == 64 && W == 8) ? 8 : 4;
   constexpr int lds_bytes = 2 * tile_bytes<D, KB>();
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&prefill_attention_kernel<D, CT, KB>),
+      reinterpret_cast<const void*>(&prefill_attention_kernel<D, CT, KB, W>),
       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
   if (attr != hipSuccess) return kvc_fail("kvc_prefill_attention: the kernel's LDS size was refused");
-  hipLaunchKernelGGL((prefill_attention_kernel<D, CT, KB>), dim3(max_pairs, nkv, nsplit), dim3(kWaves * 64),
+  // see the kernel on how block ids map to (kv head, pair)
+  const int64_t wide = (8 % nkv == 0) ? static_cast<int64_t>((max_pairs + 8 / nkv - 1) / (8 / nkv)) * 8
+                                      : (static_cast<int64_t>(max_pairs) * nkv + 7) / 8 * 8;
+  if (wide > 0x7fffffff) return kvc_fail("kvc_prefill_attention: too many blocks");
+  hipLaunchKernelGGL((prefill_attention_kernel<D, CT, KB, W>), dim3(static_cast<unsigned>(wide), 1, nsplit), dim3(W * 64),
                      lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                      q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, part_o,
                      part_ml, single);
@@ -517,19 +540,25 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
                    int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
                    float* part_o, float* part_ml, int nsplit, hipStream_t stream) {
   const int g = nh / nkv;
-  // A compute unit holds two blocks.  Tiles of 64 query rows, two a block one after the other
-  // (a late and an early one), are the fastest as long as all their blocks find room at once;
-  // more rows than that take tiles of 128 rows, which stage each key tile for twice the rows
-  // (and so does a launch that splits the keys, unless its rows are very few: its caller splits
-  // until there are blocks enough).  Few rows take one tile of 64 a block, for twice the blocks.  Measured at 32
-  // heads over 8 kv heads of 128: 1,024 tokens 43 against 47 us, 2,048 tokens 94 (pairs of
-  // 64) against 113 (pairs of 128), 3,072 tokens 165 (pairs of 128) against 217.
+  // Blocks of four waves lie two to a compute unit, blocks of eight waves one.  Tiles of 64
+  // query rows, two a block one after the other (a late and an early one), are the fastest as
+  // long as all their blocks find room at once; more rows than that take tiles of 128 rows,
+  // which stage each key tile for twice the rows (and so does a launch that splits the keys,
+  // unless its rows are very few: its caller splits until there are blocks enough).  Few rows
+  // take one tile of 64 a block, for twice the blocks.  Where the requests are long, blocks of
+  // eight waves (tiles of 128 or 256 rows) halve the loads and LDS writes per row once more.
+  // Measured at 32 heads over 8 kv heads of 128, one request, four waves against eight:
+  // 1,024 tokens 36 against 38 us, 1,536 tokens 64 against 56, 2,048 tokens 83 against 77,
+  // 3,072 tokens 149 against 144, 8,192 tokens 699 against 672; four requests of 512 tokens 29
+  // (tiles of 64 rows) and 33 (tiles of 128) against 40 (eight waves, tiles of 256).  Heads
+  // of 64: 1,024 tokens 27 against 23, 2,048 tokens 54 against 43, 8,192 tokens 445 against 393.
   // (every request but one may add a ragged tile)
   const int bq1 = 64 / g > 0 ? 64 / g : 1;
   const int tiles1 = (T + bq1 - 1) / bq1 + (R - 1);
   const int64_t pairs1 = static_cast<int64_t>((tiles1 + 1) / 2) * nkv;
   const int64_t small_tiles = static_cast<int64_t>(tiles1) * nkv;
-  int ct = 1, single = 0;
+  const bool long_requests = T / R >= (D == 64 ? 512 : 1024);
+  int ct = 1, single = 0, waves = 4;
   if (g > 64) {
     ct = 2;
   } else if (nsplit > 1) {
@@ -538,22 +567,35 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
     if (small_tiles <= 128) single = 1; else ct = 2;
   } else if (pairs1 > 512) {
     ct = 2;
-  } else if (pairs1 <= 256) {
+    if (long_requests) waves = 8;
+  } else if (pairs1 > 256) {
+    if (long_requests) {
+      waves = 8;
+      single = pairs1 <= 448;
+    }
+  } else {
     single = 1;
+    if (D == 64 && pairs1 > 128 && long_requests) waves = 8;
   }
-  // KVC_PREFILL_MODE = 1p | 1s | 2p overrides the choice for tuning
+  // KVC_PREFILL_MODE = 1p | 1s | 2p | 2s, then 4 or 8 (waves), overrides the choice for tuning
   static const char* mode = getenv("KVC_PREFILL_MODE");
   if (mode && (mode[0] == '1' || mode[0] == '2')) {
     ct = mode[0] == '2' ? 2 : 1;
     single = mode[1] == 's';
+    waves = (mode[1] && mode[2] == '8') ? 8 : 4;
   }
-  if (ct == 2)
-    return launch_prefill_ct<D, 2>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
-                                   q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window,
-                                   part_o, part_ml, nsplit, single, stream);
-  return launch_prefill_ct<D, 1>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
-                                 q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window,
-                                 part_o, part_ml, nsplit, single, stream);
+  if (g > 16 * waves * ct) return kvc_fail("kvc_prefill_attention: too many query heads per kv head");
+#define KVC_LAUNCH_PREFILL(CT_, W_)                                                                      \
+  return launch_prefill_ct<D, CT_, W_>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions, \
+                                       q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window, \
+                                       part_o, part_ml, nsplit, single, stream)
+  if (waves == 8) {
+    if (ct == 2) KVC_LAUNCH_PREFILL(2, 8);
+    KVC_LAUNCH_PREFILL(1, 8);
+  }
+  if (ct == 2) KVC_LAUNCH_PREFILL(2, 4);
+  KVC_LAUNCH_PREFILL(1, 4);
+#undef KVC_LAUNCH_PREFILL
 }
 
 }  // namespace

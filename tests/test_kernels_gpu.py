@@ -1011,11 +1011,16 @@ def test_decode_attention_long_context(ops, nsplit):
 
 
 @pytest.mark.parametrize("nh,nkv,d,whole,nsplit", [(8, 2, 128, 2100, 1), (8, 1, 64, 2100, 1), (32, 8, 128, 4200, 1),
-                                                   (8, 2, 128, 2100, 7), (8, 1, 64, 2100, 2)])
+                                                   (8, 2, 128, 2100, 7), (8, 1, 64, 2100, 2),
+                                                   (16, 4, 128, 2100, 1), (16, 4, 128, 3100, 1),
+                                                   (12, 6, 128, 2100, 1), (16, 4, 64, 4200, 1)])
 def test_prefill_attention_long_context_and_many_tokens(ops, nh, nkv, d, whole, nsplit):
     """A portion of 700 tokens after 6,000 others, and a whole prompt of thousands of tokens:
     hundreds of key tiles; the third case has enough tokens and kv heads that the kernel takes
-    its larger query tiles, the last two deal each tile's keys to several blocks."""
+    its larger query tiles, the fourth and fifth deal each tile's keys to several blocks, and
+    the last four take blocks of eight waves (one tile a block, a late and an early tile a
+    block, six kv heads, which the eight dies do not share out evenly, and heads of 64 with
+    their tiles of 128 keys)."""
     dtype, page = torch.bfloat16, 16
     seq_lens = [6700, whole]
     q_lens = [700, whole]
