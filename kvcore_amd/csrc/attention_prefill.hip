@@ -511,11 +511,12 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
   const int bq = (16 * W * CT) / g;
   // every request may end in a ragged tile and have an odd number of tiles
   const int max_pairs = single ? (T + bq - 1) / bq + R : ((T + bq - 1) / bq + R) / 2 + R;
-  // key tiles of 64 (tiles of 32, with which more blocks would fit a compute unit, were slower:
-  // 2,048 tokens 121 against 90 us)
-  // (eight waves on heads of 64 take tiles of 128 keys, so that a thread still stages whole
-  // pairs of key blocks)
-  constexpr int KB = (D == 64 && W == 8) ? 8 : 4;
+  // key tiles of 64 for four waves (tiles of 32, with which more blocks would fit a compute
+  // unit, were slower: 2,048 tokens 121 against 90 us); a block of eight waves has the compute
+  // unit's LDS to itself and takes tiles of 128 keys: half the barriers and page lookups per key
+  // (16,384 tokens 2.52 against 2.39 ms), and on heads of 64 a thread then still stages whole
+  // pairs of key blocks
+  constexpr int KB = (W == 8) ? 8 : 4;
   constexpr int lds_bytes = 2 * tile_bytes<D, KB>();
   static const hipError_t attr = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&prefill_attention_kernel<D, CT, KB, W>),
@@ -564,7 +565,12 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
   } else if (nsplit > 1) {
     // very few rows: small tiles one a block reach the blocks wanted with a quarter of the
     // splits (128 rows at 1,024 keys: 21 against 39 us)
-    if (small_tiles <= 128) single = 1; else ct = 2;
+    if (small_tiles <= 128) {
+      single = 1;
+    } else {
+      ct = 2;
+      if (long_requests) waves = 8;  // 2,048 tokens after 30,000: 1.38 against 1.32 ms
+    }
   } else if (pairs1 > 512) {
     ct = 2;
     if (long_requests) waves = 8;
