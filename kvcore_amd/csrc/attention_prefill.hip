@@ -63,7 +63,8 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
     const int32_t* __restrict__ table, int table_stride, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int num_reqs, int nh,
     int nkv, int page_size, int num_pages, float scale_log2e, int window,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int single) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, int single,
+    const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim, int interleaved) {
   constexpr int kKeyBlocks = KB;
   constexpr int NJ = D / 16;
   constexpr int NC = D / 32;
@@ -160,6 +161,55 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) qb[ct][c][e] = static_cast<__bf16>(0.f);
+      }
+    }
+    // With tables the queries arrive unrotated and are rotated here, in registers, exactly as
+    // the kernel that rotates in memory would have (float32 products, rounded once): a lane
+    // holds both elements of every pair, since rot_dim is a multiple of 64 (of 32 for
+    // neighbouring pairs).  The query rows then need not be written and read again.
+    if (cos_tab != nullptr && live[ct]) {
+      const int half = rot_dim >> 1;
+      const float* cs = cos_tab + static_cast<int64_t>(my_tok[ct]) * half;
+      const float* sn = sin_tab + static_cast<int64_t>(my_tok[ct]) * half;
+      if (interleaved) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          if (32 * c < rot_dim) {  // uniform
+            const int j0 = 16 * c + 4 * quad;
+            const f32x4_t cv = *reinterpret_cast<const f32x4_t*>(cs + j0);
+            const f32x4_t sv = *reinterpret_cast<const f32x4_t*>(sn + j0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float x0 = static_cast<float>(qb[ct][c][2 * e]);
+              const float x1 = static_cast<float>(qb[ct][c][2 * e + 1]);
+              qb[ct][c][2 * e] = static_cast<__bf16>(rotate_first(x0, x1, cv[e], sv[e]));
+              qb[ct][c][2 * e + 1] = static_cast<__bf16>(rotate_second(x0, x1, cv[e], sv[e]));
+            }
+          }
+        }
+      } else {
+        // element j < half pairs with j + half: register c with register c + half / 32
+#pragma unroll
+        for (int span = 1; span <= NC / 2; ++span) {
+          if (half == 32 * span) {  // uniform
+#pragma unroll
+            for (int c = 0; c < span; ++c) {
+              const int j0 = 32 * c + 8 * quad;
+#pragma unroll
+              for (int e4 = 0; e4 < 2; ++e4) {
+                const f32x4_t cv = *reinterpret_cast<const f32x4_t*>(cs + j0 + 4 * e4);
+                const f32x4_t sv = *reinterpret_cast<const f32x4_t*>(sn + j0 + 4 * e4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  const float x0 = static_cast<float>(qb[ct][c][4 * e4 + e]);
+                  const float x1 = static_cast<float>(qb[ct][c + span][4 * e4 + e]);
+                  qb[ct][c][4 * e4 + e] = static_cast<__bf16>(rotate_first(x0, x1, cv[e], sv[e]));
+                  qb[ct][c + span][4 * e4 + e] = static_cast<__bf16>(rotate_second(x0, x1, cv[e], sv[e]));
+                }
+              }
+            }
+          }
+        }
       }
     }
   }
@@ -506,7 +556,8 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
                       const bf16_t* v_cache, const int32_t* table, int table_stride,
                       const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                       int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
-                      float* part_o, float* part_ml, int nsplit, int single, hipStream_t stream) {
+                      float* part_o, float* part_ml, int nsplit, int single, const float* cos_tab,
+                      const float* sin_tab, int rot_dim, int interleaved, hipStream_t stream) {
   const int g = nh / nkv;
   const int bq = (16 * W * CT) / g;
   // every request may end in a ragged tile and have an odd number of tiles
@@ -529,7 +580,7 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
   hipLaunchKernelGGL((prefill_attention_kernel<D, CT, KB, W>), dim3(static_cast<unsigned>(wide), 1, nsplit), dim3(W * 64),
                      lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                      q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, part_o,
-                     part_ml, single);
+                     part_ml, single, cos_tab, sin_tab, rot_dim, interleaved);
   if (nsplit > 1) return launch_attention_combine(out, part_o, part_ml, static_cast<int64_t>(T) * nh, D, nsplit, stream);
   return kvc_check_launch("kvc_prefill_attention");
 }
@@ -539,7 +590,8 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
                    const bf16_t* v_cache, const int32_t* table, int table_stride,
                    const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                    int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
-                   float* part_o, float* part_ml, int nsplit, hipStream_t stream) {
+                   float* part_o, float* part_ml, int nsplit, const float* cos_tab, const float* sin_tab,
+                   int rot_dim, int interleaved, hipStream_t stream) {
   const int g = nh / nkv;
   // Blocks of four waves lie two to a compute unit, blocks of eight waves one.  Tiles of 64
   // query rows, two a block one after the other (a late and an early one), are the fastest as
@@ -594,7 +646,8 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
 #define KVC_LAUNCH_PREFILL(CT_, W_)                                                                      \
   return launch_prefill_ct<D, CT_, W_>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions, \
                                        q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window, \
-                                       part_o, part_ml, nsplit, single, stream)
+                                       part_o, part_ml, nsplit, single, cos_tab, sin_tab, rot_dim,     \
+                                       interleaved, stream)
   if (waves == 8) {
     if (ct == 2) KVC_LAUNCH_PREFILL(2, 8);
     KVC_LAUNCH_PREFILL(1, 8);
@@ -619,7 +672,9 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
                                      const int32_t* positions, const int32_t* q_start,
                                      const int32_t* slots, int T, int R, int nh, int nkv, int d,
                                      int page_size, int num_pages, float scale, int window,
-                                     void* part_o, void* part_ml, int nsplit, kvc_stream stream) {
+                                     void* part_o, void* part_ml, int nsplit, const float* cos_tab,
+                                     const float* sin_tab, int rot_dim, int interleaved,
+                                     kvc_stream stream) {
   if (!kvc_prefill_attention_supported(nh, nkv, d, page_size, 1))
     return kvc_fail("kvc_prefill_attention: unsupported shape (bfloat16, head size 64 or 128, at "
                     "most 64 query heads per kv head, page size a multiple of 16)");
@@ -631,6 +686,12 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
     return kvc_fail("kvc_prefill_attention: between 1 and 64 splits");
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr))
     return kvc_fail("kvc_prefill_attention: splits need a workspace");
+  if ((cos_tab == nullptr) != (sin_tab == nullptr))
+    return kvc_fail("kvc_prefill_attention: cosines and sines come together");
+  if (cos_tab != nullptr &&
+      (rot_dim <= 0 || rot_dim > d || rot_dim % (interleaved ? 32 : 64)))
+    return kvc_fail("kvc_prefill_attention: rotating the queries here needs rot_dim to be a multiple "
+                    "of 64 (32 for neighbouring pairs) and at most the head size");
   if (T == 0) return 0;
   float* po = static_cast<float*>(part_o);
   float* pml = static_cast<float*>(part_ml);
@@ -641,8 +702,8 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
   if (d == 64)
     return launch_prefill<64>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                               positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                              window, po, pml, nsplit, s);
+                              window, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
   return launch_prefill<128>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                              positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                             window, po, pml, nsplit, s);
+                             window, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
 }

@@ -506,7 +506,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
                                      T* __restrict__ v_cache, const float* __restrict__ cos_tab,
                                      const float* __restrict__ sin_tab, int rot_dim,
                                      int interleaved, const int32_t* __restrict__ kv_slot, int nh,
-                                     int nkv, int d, int page_size, int write_kv) {
+                                     int nkv, int d, int page_size, int write_kv, int head_begin) {
   const int t = blockIdx.x;
   const int slot = kv_slot[t];
   if (slot == -2) return;  // padding token
@@ -525,10 +525,10 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
 
   if constexpr (VEC == 8) {
     const int chunks = half / 8;
-    const int n_items = (nh + nkv) * chunks;
+    const int n_items = (nh + nkv - head_begin) * chunks;  // head_begin = nh: the keys only
     for (int w = threadIdx.x; w < n_items; w += blockDim.x) {
-      const int head = w / chunks;
-      const int j = (w - head * chunks) * 8;
+      const int head = head_begin + w / chunks;
+      const int j = (w - (head - head_begin) * chunks) * 8;
       T* hp = row + static_cast<int64_t>(head) * d;
       float x0[8], x1[8], c[8], s_[8], y0[8], y1[8];
       load8(hp + j, x0);
@@ -549,10 +549,10 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
       }
     }
   } else {
-    const int n_rot = (nh + nkv) * half;
+    const int n_rot = (nh + nkv - head_begin) * half;
     for (int w = threadIdx.x; w < n_rot; w += blockDim.x) {
-      const int head = w / half;
-      const int j = w - head * half;
+      const int head = head_begin + w / half;
+      const int j = w - (head - head_begin) * half;
       const int i0 = interleaved ? 2 * j : j;
       const int i1 = interleaved ? 2 * j + 1 : j + half;
       T* hp = row + static_cast<int64_t>(head) * d;
@@ -592,9 +592,11 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
 extern "C" int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_tab,
                                  const float* sin_tab, int rot_dim, int interleaved,
                                  const int32_t* kv_slot, int T, int nh, int nkv, int d,
-                                 int page_size, int write_kv, int dtype, kvc_stream stream) {
+                                 int page_size, int write_kv, int rotate_q, int dtype,
+                                 kvc_stream stream) {
   if (T < 0 || nh <= 0 || nkv <= 0 || d <= 0 || page_size <= 0)
     return kvc_fail("kvc_rope_kv_write: bad sizes");
+  const int head_begin = rotate_q ? 0 : nh;
   if (rot_dim < 0 || rot_dim > d || (rot_dim & 1))
     return kvc_fail("kvc_rope_kv_write: rot_dim must be even and at most the head size");
   if (T == 0) return 0;
@@ -607,14 +609,14 @@ extern "C" int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const 
         hipLaunchKernelGGL((rope_kv_write_kernel<Tp, 8>), dim3(T), dim3(256), 0, S(stream),
                            static_cast<Tp*>(qkv), static_cast<Tp*>(k_cache),
                            static_cast<Tp*>(v_cache), cos_tab, sin_tab, rot_dim, interleaved,
-                           kv_slot, nh, nkv, d, page_size, write_kv));
+                           kv_slot, nh, nkv, d, page_size, write_kv, head_begin));
   } else {
     KVC_DISPATCH_DTYPE(
         dtype, Tp,
         hipLaunchKernelGGL((rope_kv_write_kernel<Tp, 1>), dim3(T), dim3(256), 0, S(stream),
                            static_cast<Tp*>(qkv), static_cast<Tp*>(k_cache),
                            static_cast<Tp*>(v_cache), cos_tab, sin_tab, rot_dim, interleaved,
-                           kv_slot, nh, nkv, d, page_size, write_kv));
+                           kv_slot, nh, nkv, d, page_size, write_kv, head_begin));
   }
   return kvc_check_launch("kvc_rope_kv_write");
 }

@@ -66,11 +66,12 @@ int kvc_kv_slots(int32_t* kv_slot, const int32_t* positions, const int32_t* toke
 // set and kv_slot[t] >= 0, stores the rotated k and the v of token t at that slot:
 //   k_cache[page, kv_head, offset, :] and v_cache[page, kv_head, :, offset]
 //   (V pages keep the keys contiguous: the layout the matrix cores read).
-// Tokens with kv_slot == -2 are left alone.
+// Tokens with kv_slot == -2 are left alone.  Without rotate_q the q heads stay as they are
+// (for a consumer that rotates them itself, as kvc_prefill_attention can).
 int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_tab,
                       const float* sin_tab, int rot_dim, int interleaved, const int32_t* kv_slot,
-                      int T, int nh, int nkv, int d, int page_size, int write_kv, int dtype,
-                      kvc_stream stream);
+                      int T, int nh, int nkv, int d, int page_size, int write_kv, int rotate_q,
+                      int dtype, kvc_stream stream);
 
 // Attention of every token over its request's cache: token t at position p sees keys
 // max(0, p - window + 1) .. p (window <= 0: all), read through the block table.
@@ -111,13 +112,16 @@ int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* qkv
 // positions must rise by one along a request's tokens.  With nsplit > 1 the keys of every
 // tile are dealt to that many blocks (for few query rows against many keys) and a second
 // kernel joins their results; part_o [T*nh*nsplit, d] and part_ml [T*nh*nsplit, 2] float32
-// are its workspace.
+// are its workspace.  With cos_tab and sin_tab [T, rot_dim / 2] the queries come unrotated
+// and are rotated on their way in, as kvc_rope_kv_write would have (rot_dim a multiple of 64,
+// or of 32 when interleaved); without, they are taken as they are.
 int kvc_prefill_attention_supported(int nh, int nkv, int d, int page_size, int dtype);
 int kvc_prefill_attention(void* out, const void* q, int64_t q_stride, const void* k_cache,
                           const void* v_cache, const int32_t* table, int table_stride,
                           const int32_t* positions, const int32_t* q_start, const int32_t* slots,
                           int T, int R, int nh, int nkv, int d, int page_size, int num_pages,
                           float scale, int window, void* part_o, void* part_ml, int nsplit,
+                          const float* cos_tab, const float* sin_tab, int rot_dim, int interleaved,
                           kvc_stream stream);
 
 // C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) in float32 with float32 products and sums;

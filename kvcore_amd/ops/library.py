@@ -42,13 +42,14 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_to_float": [P, P, L, I, P],
         "kvc_rope_table": [P, P, P, P, I, I, P],
         "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
-        "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, P],
+        "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
         "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
                                  F, I, I, P],
         "kvc_decode_attention_waves": [I, I, I],
         "kvc_decode_attention_supported": [I, I, I, I, I],
-        "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, P, I, P],
+        "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, P, I,
+                                  P, P, I, I, P],
         "kvc_prefill_attention_supported": [I, I, I, I, I],
         "kvc_gemm_mid_slices": [I, I],
         "kvc_gemm_mid_bf16": [P, P, P, P, P, I, I, I, L, L, I, I, P],
@@ -225,9 +226,11 @@ def kv_slots(out: torch.Tensor, *, positions: torch.Tensor, token_req: torch.Ten
 
 def rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                   cos: torch.Tensor, sin: torch.Tensor, *, rot_dim: int, interleaved: bool,
-                  kv_slot: torch.Tensor, nh: int, nkv: int, d: int, write_kv: bool = True) -> None:
+                  kv_slot: torch.Tensor, nh: int, nkv: int, d: int, write_kv: bool = True,
+                  rotate_q: bool = True) -> None:
     """``k_cache`` is ``[pages, nkv, page_size, d]``, ``v_cache`` ``[pages, nkv, d, page_size]``,
-    both of the dtype of ``qkv``; ``kv_slot`` comes from ``kv_slots``."""
+    both of the dtype of ``qkv``; ``kv_slot`` comes from ``kv_slots``.  Without ``rotate_q``
+    the query heads are left as they are, for an attention kernel that rotates them itself."""
     T = qkv.shape[0]
     if qkv.shape != (T, (nh + 2 * nkv) * d):
         raise KernelError(f"rope_kv_write: qkv shape {tuple(qkv.shape)} does not fit heads")
@@ -242,7 +245,7 @@ def rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _dev(qkv, "qkv"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), rot_dim, int(interleaved),
         _dev(kv_slot, "kv_slot", torch.int32), T, nh, nkv, d, page_size, int(write_kv),
-        _code(qkv, "qkv"), _stream()), "kvc_rope_kv_write")
+        int(rotate_q), _code(qkv, "qkv"), _stream()), "kvc_rope_kv_write")
 
 
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -333,10 +336,13 @@ def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                       *, table: torch.Tensor, positions: torch.Tensor, q_start: torch.Tensor,
                       slots: torch.Tensor, num_reqs: int, nh: int, nkv: int, d: int, scale: float,
                       window: int = 0, nsplit: int = 1, part_o: torch.Tensor | None = None,
-                      part_ml: torch.Tensor | None = None) -> None:
+                      part_ml: torch.Tensor | None = None, cos: torch.Tensor | None = None,
+                      sin: torch.Tensor | None = None, rot_dim: int = 0, interleaved: bool = False) -> None:
     """bfloat16 attention of portions of prompts on the matrix cores (see the C header).
     ``nsplit > 1`` deals every tile's keys to that many blocks; ``part_o`` (float32,
-    ``T*nh*nsplit*d`` values) and ``part_ml`` (``T*nh*nsplit*2``) are then the workspace."""
+    ``T*nh*nsplit*d`` values) and ``part_ml`` (``T*nh*nsplit*2``) are then the workspace.
+    With ``cos`` and ``sin`` (``[T, rot_dim / 2]`` float32) the queries come unrotated and
+    the kernel rotates them (``prefill_attention_rotates`` says for which shapes)."""
     T = out.shape[0]
     if out.shape != (T, nh * d) or not out.is_contiguous() or out.dtype != torch.bfloat16:
         raise KernelError("prefill_attention: out must be contiguous bfloat16 [T, nh*d]")
@@ -353,12 +359,25 @@ def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                 part_ml.numel() < T * nh * nsplit * 2:
             raise KernelError("prefill_attention: the workspace for splits is missing or too small")
         po, pml = _dev(part_o, "part_o", torch.float32), _dev(part_ml, "part_ml", torch.float32)
+    cs = sn = None
+    if cos is not None:
+        if sin is None or cos.shape[0] < T or cos.shape[1] != rot_dim // 2 or sin.shape != cos.shape \
+                or not prefill_attention_rotates(rot_dim, interleaved):
+            raise KernelError("prefill_attention: rotary tables do not fit")
+        cs, sn = _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32)
     _check(load().kvc_prefill_attention(
         out.data_ptr(), q.data_ptr(), q.stride(0), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _dev(table, "table", torch.int32), table.shape[1], _dev(positions, "positions", torch.int32),
         _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), T, num_reqs,
-        nh, nkv, d, page_size, num_pages, float(scale), int(window), po, pml, int(nsplit), _stream()),
+        nh, nkv, d, page_size, num_pages, float(scale), int(window), po, pml, int(nsplit),
+        cs, sn, int(rot_dim) if cs is not None else 0, int(interleaved), _stream()),
         "kvc_prefill_attention")
+
+
+def prefill_attention_rotates(rot_dim: int, interleaved: bool) -> bool:
+    """Whether ``prefill_attention`` can rotate the queries itself: a lane of the kernel
+    must hold both elements of every rotary pair."""
+    return rot_dim > 0 and rot_dim % (32 if interleaved else 64) == 0
 
 
 def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int, who: str) -> tuple[int, int]:

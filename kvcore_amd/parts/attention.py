@@ -176,11 +176,16 @@ class PagedAttention(Mixer):
                              slots=ctx.slots, table=group.table, page_size=group.page_size,
                              num_pages=k_cache.shape[0])
                 ctx.scratch[slot_key] = kv_slot
+            on_matrix_cores = ctx.max_query_len > 1 and self.scale > 0 and ops.prefill_attention_supported(
+                self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype)
+            # the kernel for portions rotates the queries on their way in where it can, which
+            # saves writing them and reading them again
+            rotates = on_matrix_cores and ops.prefill_attention_rotates(rot_dim, interleaved)
             ops.rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim,
                               interleaved=interleaved, kv_slot=kv_slot, nh=self.num_heads,
-                              nkv=self.num_kv_heads, d=self.head_dim, write_kv=call.write_cache)
-            if ctx.max_query_len > 1 and self.scale > 0 and ops.prefill_attention_supported(
-                    self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
+                              nkv=self.num_kv_heads, d=self.head_dim, write_kv=call.write_cache,
+                              rotate_q=not rotates)
+            if on_matrix_cores:
                 # portions of prompts (single tokens may ride along): tiles of query rows per
                 # block, and several blocks per tile where few rows meet many keys
                 T = ctx.num_tokens
@@ -198,7 +203,9 @@ class PagedAttention(Mixer):
                                       positions=ctx.positions, q_start=ctx.q_start, slots=ctx.slots,
                                       num_reqs=ctx.num_reqs, nh=self.num_heads, nkv=self.num_kv_heads,
                                       d=self.head_dim, scale=self.scale, window=self.window,
-                                      nsplit=nsplit, part_o=part_o, part_ml=part_ml)
+                                      nsplit=nsplit, part_o=part_o, part_ml=part_ml,
+                                      **(dict(cos=cos, sin=sin, rot_dim=rot_dim, interleaved=interleaved)
+                                         if rotates else {}))
             else:
                 ops.paged_attention(attn, qkv, k_cache, v_cache, **common)
         if sink is not None:

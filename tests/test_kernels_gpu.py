@@ -744,6 +744,57 @@ def test_prefill_attention_far_key_and_window(ops, nsplit):
     assert torch.allclose(out.double().cpu().view(ql, nh, d), want, atol=1e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,rot_dim,interleaved", [(8, 2, 128, 128, False), (8, 2, 128, 64, False),
+                                                          (6, 3, 64, 64, False), (4, 1, 128, 96, True),
+                                                          (4, 4, 64, 32, True)])
+@pytest.mark.parametrize("nsplit", [1, 3])
+def test_prefill_attention_rotates_the_queries_like_the_separate_kernel(ops, nh, nkv, d, rot_dim, interleaved,
+                                                                        nsplit):
+    """Unrotated queries with the rotary tables give, bit for bit, what the rotation in memory
+    followed by the kernel without tables gives; the rotation without ``rotate_q`` leaves the
+    query heads alone and still rotates and stores the keys."""
+    dtype, page = torch.bfloat16, 16
+    seq_lens, q_lens = [300, 77], [130, 77]
+    kc, vc, table, _ = paged_setup(seq_lens, nkv, d, page, dtype, seed=11)
+    T = sum(q_lens)
+    qkv0 = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=12)
+    positions = torch.tensor(list(range(170, 300)) + list(range(77)), dtype=torch.int32, device=DEV)
+    token_req = torch.tensor([0] * 130 + [1] * 77, dtype=torch.int32, device=DEV)
+    q_start = torch.tensor([0, 130, T], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([1, 2], dtype=torch.int32, device=DEV)
+    inv = plain.rope_inv_freq(rot_dim, 10000.0).float().to(DEV)
+    cos = torch.empty(T, rot_dim // 2, device=DEV)
+    sin = torch.empty(T, rot_dim // 2, device=DEV)
+    ops.rope_table(cos, sin, positions, inv)
+    assert ops.prefill_attention_rotates(rot_dim, interleaved)
+    assert not ops.prefill_attention_rotates(32, False) and not ops.prefill_attention_rotates(16, True)
+    kv_slot = torch.empty(T, dtype=torch.int32, device=DEV)
+    ops.kv_slots(kv_slot, positions=positions, token_req=token_req, slots=slots, table=table,
+                 page_size=page, num_pages=kc.shape[0])
+    outs, caches = [], []
+    for fused in (False, True):
+        qkv, k2, v2 = qkv0.clone(), kc.clone(), vc.clone()
+        ops.rope_kv_write(qkv, k2, v2, cos, sin, rot_dim=rot_dim, interleaved=interleaved, kv_slot=kv_slot,
+                          nh=nh, nkv=nkv, d=d, rotate_q=not fused)
+        if fused:
+            assert torch.equal(qkv[:, :nh * d], qkv0[:, :nh * d])  # the queries were left alone
+        out = torch.full((T, nh * d), float("nan"), dtype=dtype, device=DEV)
+        extra = dict(cos=cos, sin=sin, rot_dim=rot_dim, interleaved=interleaved) if fused else {}
+        ops.prefill_attention(out, qkv, k2, v2, table=table, positions=positions, q_start=q_start,
+                              slots=slots, num_reqs=2, nh=nh, nkv=nkv, d=d, scale=d ** -0.5, nsplit=nsplit,
+                              part_o=torch.empty(T * nh * nsplit, d, device=DEV),
+                              part_ml=torch.empty(T * nh * nsplit, 2, device=DEV), **extra)
+        outs.append(out)
+        caches.append((k2, v2))
+    assert not torch.isnan(outs[0]).any()
+    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(caches[0][0].view(torch.int16), caches[1][0].view(torch.int16))  # the keys were rotated all the same
+    with pytest.raises(ops.KernelError, match="rotary tables"):
+        ops.prefill_attention(outs[0], qkv0, kc, vc, table=table, positions=positions, q_start=q_start,
+                              slots=slots, num_reqs=2, nh=nh, nkv=nkv, d=d, scale=d ** -0.5,
+                              cos=cos[:, :8].contiguous(), sin=sin[:, :8].contiguous(), rot_dim=16)
+
+
 def test_decode_attention_says_what_it_does_not_serve(ops):
     assert not ops.prefill_attention_supported(4, 2, 96, 16, torch.bfloat16)
     assert not ops.prefill_attention_supported(4, 2, 64, 8, torch.bfloat16)
