@@ -589,6 +589,110 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, T* __restrict__ k_cach
   }
 }
 
+// The same for eight consecutive tokens a block, with 16-byte accesses throughout (half-split
+// pairing, rot_dim a multiple of 16, head size a multiple of 8).  A V page keeps the keys
+// contiguous, so a token alone stores its value two bytes at a time, d * nkv stores 32 bytes
+// apart; when the block's eight tokens lie side by side in one page (a portion of a prompt
+// mostly does), a thread gathers one element of all eight and stores them together.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_tile_kernel(
+    T* __restrict__ qkv, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim,
+    const int32_t* __restrict__ kv_slot, int num_tokens, int nh, int nkv, int d, int page_size,
+    int write_kv, int head_begin) {
+  constexpr int TILE = 8;
+  const int t0 = blockIdx.x * TILE;
+  const int n_tok = (num_tokens - t0 < TILE) ? num_tokens - t0 : TILE;
+  const int half = rot_dim / 2;
+  const int64_t row_elems = static_cast<int64_t>(nh + 2 * nkv) * d;
+  const int64_t head_step = static_cast<int64_t>(page_size) * d;  // between kv heads in a page
+  const int chunks = half / 8;
+  const int n_items = (nh + nkv - head_begin) * chunks;  // head_begin = nh: the keys only
+  // ---- rotations, and the rotated keys into the cache
+  for (int w = threadIdx.x; w < n_tok * n_items; w += blockDim.x) {
+    const int ti = w / n_items;
+    const int item = w - ti * n_items;
+    const int t = t0 + ti;
+    const int slot = kv_slot[t];
+    if (slot == -2) continue;  // padding token
+    const int head = head_begin + item / chunks;
+    const int j = (item - (head - head_begin) * chunks) * 8;
+    T* hp = qkv + t * row_elems + static_cast<int64_t>(head) * d;
+    const float* cs = cos_tab + static_cast<int64_t>(t) * half;
+    const float* sn = sin_tab + static_cast<int64_t>(t) * half;
+    float x0[8], x1[8], c[8], s_[8], y0[8], y1[8];
+    load8(hp + j, x0);
+    load8(hp + j + half, x1);
+    load8(cs + j, c);
+    load8(sn + j, s_);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      y0[e] = rotate_first(x0[e], x1[e], c[e], s_[e]);
+      y1[e] = rotate_second(x0[e], x1[e], c[e], s_[e]);
+    }
+    store8(hp + j, y0);
+    store8(hp + j + half, y1);
+    if (head >= nh && write_kv && slot >= 0) {
+      const int page = slot / page_size, off = slot - page * page_size;
+      T* kc = k_cache + (static_cast<int64_t>(page) * nkv * page_size + off) * d + (head - nh) * head_step;
+      store8(kc + j, y0);
+      store8(kc + j + half, y1);
+    }
+  }
+  if (!write_kv) return;
+  // ---- k elements beyond the rotated part, eight at a time
+  const int tail_chunks = (d - rot_dim) / 8;
+  for (int w = threadIdx.x; w < n_tok * nkv * tail_chunks; w += blockDim.x) {
+    const int ti = w / (nkv * tail_chunks);
+    const int rest = w - ti * nkv * tail_chunks;
+    const int head = rest / tail_chunks;
+    const int i = rot_dim + (rest - head * tail_chunks) * 8;
+    const int slot = kv_slot[t0 + ti];
+    if (slot < 0) continue;
+    const int page = slot / page_size, off = slot - page * page_size;
+    float v[8];
+    load8(qkv + (t0 + ti) * row_elems + static_cast<int64_t>(nh + head) * d + i, v);
+    store8(k_cache + (static_cast<int64_t>(page) * nkv * page_size + off) * d + head * head_step + i, v);
+  }
+  // ---- v: element i of a head goes to V[page, head, i, off]
+  const int s0 = kv_slot[t0];
+  bool side_by_side = n_tok == TILE && s0 >= 0 && (s0 & 7) == 0 && (page_size & 7) == 0;
+  for (int ti = 1; ti < n_tok; ++ti) side_by_side = side_by_side && kv_slot[t0 + ti] == s0 + ti;
+  // (eight slots from a multiple of eight stay within a page whose size is a multiple of eight)
+  if (side_by_side) {
+    const int page = s0 / page_size, off = s0 - page * page_size;
+    const int64_t v_base = static_cast<int64_t>(page) * nkv * page_size * d + off;
+    for (int w = threadIdx.x; w < nkv * d; w += blockDim.x) {
+      const int head = w / d;
+      const int i = w - head * d;
+      const T* src = qkv + t0 * row_elems + static_cast<int64_t>(nh + nkv + head) * d + i;
+      alignas(16) T vals[TILE];
+#pragma unroll
+      for (int ti = 0; ti < TILE; ++ti) vals[ti] = src[ti * row_elems];
+      T* dst = v_cache + v_base + head * head_step + static_cast<int64_t>(i) * page_size;
+      if constexpr (sizeof(T) == 2) {
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(vals);
+      } else {
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(vals);
+        *reinterpret_cast<uint4*>(dst + 4) = *reinterpret_cast<const uint4*>(vals + 4);
+      }
+    }
+    return;
+  }
+  for (int w = threadIdx.x; w < n_tok * nkv * d; w += blockDim.x) {
+    const int ti = w / (nkv * d);
+    const int rest = w - ti * nkv * d;
+    const int head = rest / d;
+    const int i = rest - head * d;
+    const int slot = kv_slot[t0 + ti];
+    if (slot < 0) continue;
+    const int page = slot / page_size, off = slot - page * page_size;
+    v_cache[static_cast<int64_t>(page) * nkv * page_size * d + off + head * head_step +
+            static_cast<int64_t>(i) * page_size] =
+        qkv[(t0 + ti) * row_elems + static_cast<int64_t>(nh + nkv + head) * d + i];
+  }
+}
+
 extern "C" int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_tab,
                                  const float* sin_tab, int rot_dim, int interleaved,
                                  const int32_t* kv_slot, int T, int nh, int nkv, int d,
@@ -603,7 +707,15 @@ extern "C" int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const 
   const auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   const bool vec = !interleaved && rot_dim > 0 && rot_dim % 16 == 0 && d % 8 == 0 &&
                    aligned16(qkv) && aligned16(k_cache) && aligned16(cos_tab) && aligned16(sin_tab);
-  if (vec) {
+  if (vec && T >= 16 && aligned16(v_cache)) {
+    // steps of many tokens: eight tokens a block
+    KVC_DISPATCH_DTYPE(
+        dtype, Tp,
+        hipLaunchKernelGGL((rope_kv_write_tile_kernel<Tp>), dim3((T + 7) / 8), dim3(256), 0, S(stream),
+                           static_cast<Tp*>(qkv), static_cast<Tp*>(k_cache),
+                           static_cast<Tp*>(v_cache), cos_tab, sin_tab, rot_dim, kv_slot, T, nh, nkv, d,
+                           page_size, write_kv, head_begin));
+  } else if (vec) {
     KVC_DISPATCH_DTYPE(
         dtype, Tp,
         hipLaunchKernelGGL((rope_kv_write_kernel<Tp, 8>), dim3(T), dim3(256), 0, S(stream),

@@ -398,6 +398,56 @@ def test_rope_kv_write(ops, dtype, interleaved, rot_dim):
     assert torch.allclose(qkv.double().cpu().view(T, -1, d)[live, :nh], want_q[live], **tol(dtype))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,rot_dim,page", [(4, 2, 64, 64, 16), (3, 1, 32, 16, 8), (2, 2, 128, 64, 48)])
+@pytest.mark.parametrize("rotate_q", [True, False])
+def test_rope_kv_write_of_many_tokens_equals_token_by_token(ops, dtype, nh, nkv, d, rot_dim, page, rotate_q):
+    """Steps of 16 tokens and more take a kernel that handles eight tokens a block and stores
+    the values of eight neighbours in a page together.  It must leave the bits that the kernel
+    for few tokens leaves: requests that start in mid-page, a run that crosses a page, a
+    padding token, a token without a page, a ragged last block."""
+    lens = [(5, 37), (0, 9), (24, 30)]  # (first position, tokens) per request
+    positions, token_req = [], []
+    for r, (first, n) in enumerate(lens):
+        positions += list(range(first, first + n))
+        token_req += [r] * n
+    positions += [0, 20]
+    token_req += [-1, 1]  # a padding token, and one more token of request 1, apart from its others
+    T = len(positions)
+    positions = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    token_req = torch.tensor(token_req, dtype=torch.int32, device=DEV)
+    slots = torch.tensor([2, 0, 1], dtype=torch.int32, device=DEV)
+    pages_per = -(-60 // page)
+    n_pages = 3 * pages_per + 1
+    table = torch.zeros(3, pages_per + 1, dtype=torch.int32, device=DEV)
+    order = torch.randperm(n_pages - 1, generator=torch.Generator().manual_seed(3)) + 1
+    for row in range(3):
+        table[row, :pages_per] = order[row * pages_per:(row + 1) * pages_per].to(torch.int32)
+    table[1, 53 // page] = 0  # request 2 (slot 1) has no page for its last positions: they are not stored
+    kv_slot = torch.empty(T, dtype=torch.int32, device=DEV)
+    ops.kv_slots(kv_slot, positions=positions, token_req=token_req, slots=slots, table=table,
+                 page_size=page, num_pages=n_pages)
+    assert (kv_slot == -1).any() and (kv_slot == -2).any()
+    inv = plain.rope_inv_freq(rot_dim, 10000.0).float().to(DEV)
+    cos = torch.empty(T, rot_dim // 2, device=DEV)
+    sin = torch.empty(T, rot_dim // 2, device=DEV)
+    ops.rope_table(cos, sin, positions, inv)
+    qkv0 = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=4)
+    results = []
+    for step in (T, 7):  # all at once, then seven tokens a call
+        qkv = qkv0.clone()
+        kc, vc = make_cache(n_pages, nkv, page, d, dtype)
+        for a in range(0, T, step):
+            b = min(a + step, T)
+            ops.rope_kv_write(qkv[a:b], kc, vc, cos[a:b], sin[a:b], rot_dim=rot_dim, interleaved=False,
+                              kv_slot=kv_slot[a:b], nh=nh, nkv=nkv, d=d, rotate_q=rotate_q)
+        results.append((qkv, kc, vc))
+    bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+    for one, other in zip(results[0], results[1]):
+        assert torch.equal(one.view(bits), other.view(bits))
+    assert not torch.isnan(results[0][1]).all() and torch.isnan(results[0][1]).any()
+
+
 def test_kv_slots_vector_of_the_reference(ops):
     """tests/test_block_table.py:65-85: rows [3,4] and [5], page size 2, positions
     [0,1,2,3,0,1] -> slots [6,7,8,9,10,11]; beyond the row's pages there is no slot."""
