@@ -446,3 +446,49 @@ def test_layer_sizes_of_the_8b_model(tmp_path):
     got = collect(session, steps)
     rms = float(torch.cat([e.flatten() for e in expect.values()]).pow(2).mean().sqrt())
     compare(got, expect, torch.bfloat16, logit_rms=rms)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_configurations(tmp_path, seed):
+    """Configurations drawn at random (head sizes in steps of 16, any head counts and groups,
+    widths, feed-forward widths and vocabularies that are no power of two, pages of 8 to 48
+    tokens, with and without biases, tied head and scaled rotation): whole requests and mixed
+    batches with page reuse, in both dtypes, against the plain implementation."""
+    import random
+
+    from tests import helpers
+
+    rng = random.Random(1000 + seed)
+    d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+    nkv = rng.choice([1, 2, 3, 4, 5])
+    nh = nkv * rng.choice([1, 2, 3, 4, 7])
+    vocab = rng.choice([97, 300, 515, 1000])
+    page = rng.choice([8, 16, 32, 48])
+    config = {
+        "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": rng.choice([1, 2, 3]),
+        "hidden_size": rng.choice([40, 56, 72, 100, 136, 200, 264]), "num_attention_heads": nh,
+        "num_key_value_heads": nkv, "head_dim": d, "intermediate_size": rng.choice([88, 120, 200, 301, 512]),
+        "vocab_size": vocab, "rope_theta": rng.choice([1e4, 5e5]),
+        "rope_scaling": rng.choice([None, {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                           "high_freq_factor": 4.0, "original_max_position_embeddings": 64}]),
+        "tie_word_embeddings": rng.random() < 0.5, "rms_norm_eps": rng.choice([1e-5, 1e-6]),
+        "max_position_embeddings": 512, "hidden_act": "silu", "attention_bias": rng.random() < 0.3,
+        "mlp_bias": rng.random() < 0.3,
+    }
+    folder = make_model_dir(tmp_path, config, seed=seed)
+    cfg, weights = plain.load_model_folder(folder)
+    token_lists = {f"q{i}": random_tokens(rng.randint(1, 90) + EXTRA, vocab, seed=seed * 10 + i) for i in range(6)}
+    expect = {rid: plain.llama_forward(cfg, weights, t, dtype=torch.float64) for rid, t in token_lists.items()}
+    rms = max(float(torch.cat([e.flatten() for e in expect.values()]).pow(2).mean().sqrt()), helpers.TINY_LOGIT_RMS)
+    for dtype in DTYPES:
+        for rid, t in list(token_lists.items())[:2]:
+            session = session_for(folder, dtype, page, max_tokens=len(t))
+            got = collect(session, [{"step": 0, "entries": [{"id": rid, "tokens": t, "want": list(range(len(t)))}],
+                                     "end": [rid]}])
+            compare(got, expect, dtype, logit_rms=rms)
+        rounded = sorted((-(-len(t) // 64) * 64 for t in token_lists.values()), reverse=True)
+        session = session_for(folder, dtype, page, max_tokens=sum(rounded[:4]))
+        got = collect(session, mixed_trace(token_lists, seed=seed))
+        assert len(got) == sum(len(t) for t in token_lists.values())
+        compare(got, expect, dtype, logit_rms=rms)
+        assert session.manager.num_free_pages()[0] == session.num_pages - 1
