@@ -30,8 +30,8 @@ def folders(tmp_path_factory):
 
 
 def make_engine(folder, dtype, page, *, num_pages=None, max_seqs=4, budget=64, partial=4, threshold=0,
-                run_ahead=True):
-    from kvcore_amd import (CacheConfig, KVCoreConfig, LoadConfig, ModelConfig, SchedulerConfig)
+                run_ahead=True, graphs=True):
+    from kvcore_amd import (CacheConfig, DeviceConfig, KVCoreConfig, LoadConfig, ModelConfig, SchedulerConfig)
     from kvcore_amd.engine.llm_engine import LLMEngine
 
     return LLMEngine(KVCoreConfig(
@@ -42,6 +42,7 @@ def make_engine(folder, dtype, page, *, num_pages=None, max_seqs=4, budget=64, p
                                          max_num_partial_prefills=partial, max_long_partial_prefills=partial,
                                          long_prefill_token_threshold=threshold,
                                          decode_run_ahead=run_ahead),
+        device_config=DeviceConfig(use_hip_graphs=graphs),
     ))
 
 
@@ -145,8 +146,8 @@ def test_steps_launched_ahead_give_the_tokens_of_steps_taken_one_by_one(folders,
     prompts = {f"r{i}": random_tokens(n, 256, seed=500 + i) for i, n in enumerate((9, 17, 30, 5, 12))}
     caps = {"r0": 40, "r1": 23, "r2": 40, "r3": 31, "r4": 12}
 
-    def run(run_ahead, stop):
-        engine = make_engine(folder, dtype, page, run_ahead=run_ahead, max_seqs=4)
+    def run(run_ahead, stop, graphs=True):
+        engine = make_engine(folder, dtype, page, run_ahead=run_ahead, max_seqs=4, graphs=graphs)
         engine.engine_core.stop_token_ids = set(stop)
         launched = 0
         core = engine.engine_core
@@ -176,6 +177,9 @@ def test_steps_launched_ahead_give_the_tokens_of_steps_taken_one_by_one(folders,
     assert none_ahead == 0 and ahead > 10
     assert any(reason.value == "stop" for _, reason in want.values())
     assert got == want
+    if dtype == "float32":  # and launch by launch, without captured graphs
+        plain_launches, ahead = run(True, stop, graphs=False)
+        assert ahead > 10 and plain_launches == want
 
 
 def test_abort_while_a_step_is_in_flight(folders):
