@@ -71,6 +71,9 @@ def parse_args():
                    help="time to the first token of one N-token prompt, in portions of 2,048 "
                         "tokens; prints its own line")
     p.add_argument("--page-size", type=int, default=PAGE_SIZE, help="tokens a cache page")
+    p.add_argument("--pack-weights", action=argparse.BooleanOptionalAction, default=None,
+                   help="second copy of the weights in the order decode steps stream them "
+                        "(default: where the device has room, as the engine decides)")
     p.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     p.add_argument("--only-prefill", action="store_true",
                    help="run only the 2,048-token prefill (for profiling); prints its own line")
@@ -121,7 +124,8 @@ def main() -> int:
     torch.cuda.set_device(0)
 
     t0 = time.perf_counter()
-    model = build_model(".", dtype, device, load_format="random", seed=0, config_override=cfg)
+    model = build_model(".", dtype, device, load_format="random", seed=0, config_override=cfg,
+                        pack_weights=args.pack_weights)
     print(f"[bench] model built in {time.perf_counter() - t0:.1f} s, "
           f"{model.num_param_bytes() / 2**30:.2f} GiB", file=sys.stderr, flush=True)
 

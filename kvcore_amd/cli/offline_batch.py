@@ -47,6 +47,9 @@ def parse_args(argv=None) -> argparse.Namespace:
     p.add_argument("--decode-run-ahead", action=argparse.BooleanOptionalAction, default=True,
                    help="while requests only decode, launch the next step before the tokens of the "
                         "step in flight have reached the host")
+    p.add_argument("--pack-decode-weights", action=argparse.BooleanOptionalAction, default=None,
+                   help="keep a second copy of the weight matrices in the order decode steps stream "
+                        "them (default: where the device has room)")
     p.add_argument("--num-gpu-blocks", type=int, default=None)
     p.add_argument("--gpu-memory-utilization", type=float, default=0.9)
     p.add_argument("--random-weights", action="store_true",
@@ -108,7 +111,7 @@ def build_config(args: argparse.Namespace):
         model_config=ModelConfig(model=str(Path(args.model).expanduser()), dtype=args.dtype,
                                  max_model_len=args.max_model_len, attn_backend=args.attn_backend),
         load_config=LoadConfig(load_format="random" if args.random_weights else "safetensors",
-                               seed=args.seed),
+                               seed=args.seed, pack_decode_weights=args.pack_decode_weights),
         cache_config=CacheConfig(block_size=args.block_size, num_gpu_blocks=args.num_gpu_blocks,
                                  gpu_memory_utilization=args.gpu_memory_utilization),
         scheduler_config=SchedulerConfig(

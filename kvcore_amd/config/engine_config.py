@@ -59,11 +59,15 @@ class LoadConfig:
     """Reference: config.py:33-40.  ``load_format`` is ``"safetensors"`` (read the
     folder's files) or ``"random"`` (fill every parameter from ``seed``; the folder
     then needs only config.json).  ``strict`` also refuses unexpected tensors, which
-    the reference drops silently (kvcore/model/model_utils.py:65-76)."""
+    the reference drops silently (kvcore/model/model_utils.py:65-76).
+    ``pack_decode_weights``: keep a second copy of the bfloat16 weight matrices in the order
+    in which decode steps of few tokens stream them (``ops.pack_weight``: some 6% off such a
+    step for twice the weights' memory); None decides by the room on the device."""
 
     load_format: str = "safetensors"
     strict: bool = True
     seed: int = 0
+    pack_decode_weights: bool | None = None
 
     def __post_init__(self) -> None:
         if self.load_format not in ("safetensors", "random", "auto"):

@@ -54,7 +54,7 @@ template <int RT, int NT, int U, int MAXW, typename OutT, bool GATED, int FOLD =
 __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict__ C, const bf16_t* __restrict__ A,
                                    const bf16_t* __restrict__ W, const bf16_t* __restrict__ bias,
                                    int M, int N, int K, int64_t lda, int64_t ldc, int k_per_wave,
-                                   const SkinnyExtras ex) {
+                                   const SkinnyExtras ex, int packed) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
   extern __shared__ float red[];  // [waves - 1][RT * NT][64][4], then 16 row scales and [16][256] parts of their sums if FOLD & 1
   // wave-uniform values are made scalar on purpose: a condition on them becomes a scalar
@@ -69,12 +69,16 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
   const int k_begin = wave * k_per_wave;
   const int k_end = (k_begin + k_per_wave < K) ? k_begin + k_per_wave : K;
 
+  const int ks = packed ? 16 : 1;  // elements between a row's 32-wide steps, in units of 32
   const bf16_t* wp[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const int r = GATED ? n0 + col : n0 + rt * 16 + col;
     const int64_t row = (r < N ? r : N - 1) + ((GATED && rt == 1) ? N : 0);
-    wp[rt] = W + row * K + 8 * quad;
+    // packed: tiles of 16 rows x 32 k stored one after the other along K, so that the 64 lanes
+    // of a load read 1 KB in one piece (see kvc_pack_weight)
+    wp[rt] = packed ? W + (row >> 4) * (static_cast<int64_t>(K) * 16) + (row & 15) * 32 + 8 * quad
+                    : W + row * K + 8 * quad;
   }
   const bf16_t* ap[NT];
   bool tok_ok[NT];
@@ -124,8 +128,8 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
     const int k = k_begin + 64 * step;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      abuf[stage][rt][0] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k);
-      abuf[stage][rt][1] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k + 32);
+      abuf[stage][rt][0] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + static_cast<int64_t>(k) * ks);
+      abuf[stage][rt][1] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + static_cast<int64_t>(k + 32) * ks);
     }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -233,7 +237,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
   for (; k < k_full; k += 32) {
     bf16x8_t a[RT], b[NT];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) a[rt] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k);
+    for (int rt = 0; rt < RT; ++rt) a[rt] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + static_cast<int64_t>(k) * ks);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) b[nt] = *reinterpret_cast<const bf16x8_t*>(ap[nt] + k);
 #pragma unroll
@@ -247,7 +251,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
     bf16x8_t a[RT], b[NT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
-      a[rt] = valid ? *reinterpret_cast<const bf16x8_t*>(wp[rt] + k_full) : zero8();
+      a[rt] = valid ? *reinterpret_cast<const bf16x8_t*>(wp[rt] + static_cast<int64_t>(k_full) * ks) : zero8();
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
       b[nt] = valid ? *reinterpret_cast<const bf16x8_t*>(ap[nt] + k_full) : zero8();
@@ -384,7 +388,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
 
 template <int RT, int NT, typename OutT, bool GATED = false>
 void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
-            int64_t lda, int64_t ldc, int waves, int k_per_wave, const SkinnyExtras& ex,
+            int64_t lda, int64_t ldc, int waves, int k_per_wave, const SkinnyExtras& ex, int packed,
             hipStream_t stream) {
   // steps in flight by what fits in registers beside the accumulators
   constexpr int STAGES = (RT + NT <= 5) ? 4 : ((RT + NT <= 6) ? 3 : 2);
@@ -396,7 +400,7 @@ void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M
   const int fold = (ex.in_ss != nullptr ? 1 : 0) | (ex.residual != nullptr ? 2 : 0);
 #define KVC_SKINNY_LAUNCH(FOLD_)                                                                   \
   hipLaunchKernelGGL((gemm_skinny_kernel<RT, NT, STAGES, MAXW, OutT, GATED, FOLD_>), grid, block, \
-                     lds, stream, C, A, W, bias, M, N, K, lda, ldc, k_per_wave, ex)
+                     lds, stream, C, A, W, bias, M, N, K, lda, ldc, k_per_wave, ex, packed)
   if constexpr (NT == 1 && sizeof(OutT) == 2) {  // folded norms are for steps of few rows
     switch (fold) {
       case 0: KVC_SKINNY_LAUNCH(0); break;
@@ -436,14 +440,14 @@ inline void pick_shape(int N, int K, int* rt_out, int* waves_out) {
 
 template <typename OutT>
 int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
-             int64_t lda, int64_t ldc, const SkinnyExtras& ex, hipStream_t stream) {
+             int64_t lda, int64_t ldc, const SkinnyExtras& ex, int packed, hipStream_t stream) {
   int rt, waves;
   pick_shape(N, K, &rt, &waves);
   const int nt = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 63) / 64 * 64;
 #define KVC_SKINNY(RT_, NT_) \
-  launch<RT_, NT_, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, ex, stream)
+  launch<RT_, NT_, OutT>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, ex, packed, stream)
   switch (rt * 10 + nt) {
     case 11: KVC_SKINNY(1, 1); break;
     case 12: KVC_SKINNY(1, 2); break;
@@ -459,14 +463,14 @@ int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int 
 
 // silu(A Wg^T) * (A Wu^T) with Wg the first N rows of W and Wu the next N
 int dispatch_gated(bf16_t* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N,
-                   int K, int64_t lda, int64_t ldc, const SkinnyExtras& ex, hipStream_t stream) {
+                   int K, int64_t lda, int64_t ldc, const SkinnyExtras& ex, int packed, hipStream_t stream) {
   int waves = 4;
   while (waves > 1 && K / waves < 128) waves /= 2;
   const int nt = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 63) / 64 * 64;
 #define KVC_SKINNY_GATED(NT_) \
-  launch<2, NT_, bf16_t, true>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, ex, stream)
+  launch<2, NT_, bf16_t, true>(C, A, W, bias, M, N, K, lda, ldc, waves, k_per_wave, ex, packed, stream)
   switch (nt) {
     case 1: KVC_SKINNY_GATED(1); break;
     case 2: KVC_SKINNY_GATED(2); break;
@@ -482,7 +486,7 @@ int dispatch_gated(bf16_t* C, const bf16_t* A, const bf16_t* W, const bf16_t* bi
 namespace {
 
 int check_operands(const char* who, const void* A, const void* W, int M, int N, int K, int64_t lda,
-                   int64_t ldc) {
+                   int64_t ldc, int packed) {
   static thread_local char msg[160];
   if (M < 0 || M > 64 || N <= 0 || K <= 0 || lda < K || ldc < N) {
     snprintf(msg, sizeof(msg), "%s: bad sizes (1 to 64 rows)", who);
@@ -490,6 +494,10 @@ int check_operands(const char* who, const void* A, const void* W, int M, int N, 
   }
   if (K % 8 || lda % 8) {
     snprintf(msg, sizeof(msg), "%s: K and the row stride must be multiples of 8", who);
+    return kvc_fail(msg);
+  }
+  if (packed && (N % 16 || K % 64)) {
+    snprintf(msg, sizeof(msg), "%s: packed weights have a multiple of 16 rows of a multiple of 64", who);
     return kvc_fail(msg);
   }
   if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15)) {
@@ -505,29 +513,57 @@ const SkinnyExtras kNoExtras = {nullptr, 0, 1.f, 0.f, nullptr, 0, nullptr, nullp
 
 extern "C" int kvc_gemm_skinny_silu_mul_bf16(void* C, const void* A, const void* W, const void* bias,
                                              int M, int N, int K, int64_t lda, int64_t ldc,
-                                             kvc_stream stream) {
-  if (int rc = check_operands("kvc_gemm_skinny_silu_mul_bf16", A, W, M, N, K, lda, ldc)) return rc;
+                                             int packed, kvc_stream stream) {
+  if (int rc = check_operands("kvc_gemm_skinny_silu_mul_bf16", A, W, M, N, K, lda, ldc, packed)) return rc;
   if (M == 0) return 0;
   return dispatch_gated(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
                         static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N, K,
-                        lda, ldc, kNoExtras, reinterpret_cast<hipStream_t>(stream));
+                        lda, ldc, kNoExtras, packed, reinterpret_cast<hipStream_t>(stream));
 }
 
 extern "C" int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M,
                                     int N, int K, int64_t lda, int64_t ldc, int out_dtype,
-                                    kvc_stream stream) {
-  if (int rc = check_operands("kvc_gemm_skinny_bf16", A, W, M, N, K, lda, ldc)) return rc;
+                                    int packed, kvc_stream stream) {
+  if (int rc = check_operands("kvc_gemm_skinny_bf16", A, W, M, N, K, lda, ldc, packed)) return rc;
   if (M == 0) return 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (out_dtype == 0)
     return dispatch<float>(static_cast<float*>(C), static_cast<const bf16_t*>(A),
                            static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N,
-                           K, lda, ldc, kNoExtras, s);
+                           K, lda, ldc, kNoExtras, packed, s);
   if (out_dtype == 1)
     return dispatch<bf16_t>(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
                             static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N,
-                            K, lda, ldc, kNoExtras, s);
+                            K, lda, ldc, kNoExtras, packed, s);
   return kvc_fail("kvc_gemm_skinny_bf16: unknown output dtype code");
+}
+
+namespace {
+
+// dst tile (n / 16, k / 32) holds src[16 rows][32 k] in one piece of 1 KB, the tiles of a row
+// block one after the other along K
+__global__ void pack_weight_kernel(bf16_t* __restrict__ dst, const bf16_t* __restrict__ src, int N, int K) {
+  const int64_t piece = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;  // 8 elements
+  const int per_row = K / 8;
+  if (piece >= static_cast<int64_t>(N) * per_row) return;
+  const int n = static_cast<int>(piece / per_row);
+  const int k = static_cast<int>(piece % per_row) * 8;
+  const int64_t at = (static_cast<int64_t>(n >> 4) * (K / 32) + (k >> 5)) * 512 + (n & 15) * 32 + (k & 31);
+  *reinterpret_cast<uint4*>(dst + at) = *reinterpret_cast<const uint4*>(src + static_cast<int64_t>(n) * K + k);
+}
+
+}  // namespace
+
+extern "C" int kvc_pack_weight(void* dst, const void* src, int N, int K, kvc_stream stream) {
+  if (N <= 0 || K <= 0 || N % 16 || K % 64)
+    return kvc_fail("kvc_pack_weight: a multiple of 16 rows of a multiple of 64");
+  if ((reinterpret_cast<uintptr_t>(dst) & 15) || (reinterpret_cast<uintptr_t>(src) & 15) || dst == src)
+    return kvc_fail("kvc_pack_weight: two different 16-byte aligned matrices");
+  const int64_t pieces = static_cast<int64_t>(N) * (K / 8);
+  hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>((pieces + 255) / 256)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), static_cast<bf16_t*>(dst),
+                     static_cast<const bf16_t*>(src), N, K);
+  return kvc_check_launch("kvc_pack_weight");
 }
 
 extern "C" int kvc_gemm_skinny_blocks(int N, int K, int gated) {
@@ -542,8 +578,9 @@ extern "C" int kvc_gemm_skinny_fused_bf16(void* C, const void* A, const void* W,
                                           int M, int N, int K, int64_t lda, int64_t ldc, int gated,
                                           const float* in_ss, int in_parts, int in_width,
                                           float in_eps, float* residual, int64_t ldr,
-                                          const float* gain, float* out_ss, kvc_stream stream) {
-  if (int rc = check_operands("kvc_gemm_skinny_fused_bf16", A, W, M, N, K, lda, ldc)) return rc;
+                                          const float* gain, float* out_ss, int packed,
+                                          kvc_stream stream) {
+  if (int rc = check_operands("kvc_gemm_skinny_fused_bf16", A, W, M, N, K, lda, ldc, packed)) return rc;
   if ((in_ss != nullptr || residual != nullptr) && M > 16)
     return kvc_fail("kvc_gemm_skinny_fused_bf16: norms are folded in for at most 16 rows");
   if (in_ss != nullptr && (in_parts <= 0 || in_width <= 0))
@@ -558,8 +595,8 @@ extern "C" int kvc_gemm_skinny_fused_bf16(void* C, const void* A, const void* W,
   if (gated)
     return dispatch_gated(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
                           static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N, K,
-                          lda, ldc, ex, s);
+                          lda, ldc, ex, packed, s);
   return dispatch<bf16_t>(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
                           static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N, K,
-                          lda, ldc, ex, s);
+                          lda, ldc, ex, packed, s);
 }

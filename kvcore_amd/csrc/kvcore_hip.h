@@ -143,16 +143,27 @@ int kvc_gemm_mid_bf16(void* C, void* partial, const void* A, const void* W, cons
 
 // C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) for M <= 64 rows of bfloat16 on the matrix
 // cores, float32 sums, weights streamed once; C is float32 (out_dtype 0) or bfloat16 (1).
-// K and lda must be multiples of 8, A and W 16-byte aligned.
+// K and lda must be multiples of 8, A and W 16-byte aligned.  With `packed` W is what
+// kvc_pack_weight made of the matrix (N a multiple of 16, K of 64): the same sums in the same
+// order, read in contiguous kilobytes.
 int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
-                         int K, int64_t lda, int64_t ldc, int out_dtype, kvc_stream stream);
+                         int K, int64_t lda, int64_t ldc, int out_dtype, int packed,
+                         kvc_stream stream);
+
+// dst = src [N, K] bfloat16 in tiles of 16 rows x 32 columns of 1 KB each, the tiles of 16
+// rows one after the other along K (N a multiple of 16, K of 64): element (n, k) goes to
+// ((n / 16) * (K / 32) + k / 32) * 512 + (n % 16) * 32 + k % 32.  That is the order in which
+// the products for few rows read the weights, whose loads then are one contiguous kilobyte
+// instead of 64 bytes from each of 16 rows.
+int kvc_pack_weight(void* dst, const void* src, int N, int K, kvc_stream stream);
 
 // C[M, N] = silu(A Wg^T + bg) * (A Wu^T + bu) for M <= 64 rows of bfloat16, where Wg is rows
 // 0..N-1 of W[2N, K] and Wu rows N..2N-1 (bias[2N] likewise): the gated feed-forward's first
 // product with its activation, both factors rounded to bfloat16 before the activation as the
 // two-kernel form stores them.  C is bfloat16.
 int kvc_gemm_skinny_silu_mul_bf16(void* C, const void* A, const void* W, const void* bias, int M,
-                                  int N, int K, int64_t lda, int64_t ldc, kvc_stream stream);
+                                  int N, int K, int64_t lda, int64_t ldc, int packed,
+                                  kvc_stream stream);
 
 // The same products with the RMS norm of the rows folded in, for steps of at most 16 tokens,
 // so that no separate norm kernel runs between them:
@@ -168,7 +179,8 @@ int kvc_gemm_skinny_blocks(int N, int K, int gated);
 int kvc_gemm_skinny_fused_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
                                int K, int64_t lda, int64_t ldc, int gated, const float* in_ss,
                                int in_parts, int in_width, float in_eps, float* residual,
-                               int64_t ldr, const float* gain, float* out_ss, kvc_stream stream);
+                               int64_t ldr, const float* gain, float* out_ss, int packed,
+                               kvc_stream stream);
 
 // table[triples[3i], triples[3i+1]] = triples[3i+2] for i < n.
 int kvc_table_update(int32_t* table, int table_stride, int table_rows, const int32_t* triples,

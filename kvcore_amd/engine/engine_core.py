@@ -79,7 +79,8 @@ class EngineCore:
             fmt = config.load_config.load_format
             model = build_model(config.model_config.model, self.dtype, device,
                                 load_format="random" if fmt == "random" else "safetensors",
-                                seed=config.load_config.seed, strict=config.load_config.strict)
+                                seed=config.load_config.seed, strict=config.load_config.strict,
+                                pack_weights=config.load_config.pack_decode_weights)
         self.model = model
         logger.info("model ready in %.2f s (%d parameter bytes)", time.perf_counter() - t0,
                     model.num_param_bytes())

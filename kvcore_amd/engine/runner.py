@@ -65,9 +65,10 @@ class StepOutput:
 
 def build_model(model_dir: str | Path, dtype: torch.dtype, device: str | torch.device,
                 *, load_format: str = "safetensors", seed: int = 0, strict: bool = True,
-                config_override: dict | None = None) -> DecoderModel:
+                config_override: dict | None = None, pack_weights: bool | None = None) -> DecoderModel:
     """config.json -> registry -> spec -> model with weights.  ``load_format="random"``
-    fills the parameters from ``seed`` instead of reading weight files."""
+    fills the parameters from ``seed`` instead of reading weight files.  ``pack_weights``:
+    see ``DecoderModel.pack_product_weights`` (None: where there is room)."""
     from kvcore_amd.weights.loader import init_random_weights, load_weights
 
     config = config_override if config_override is not None else read_config_json(model_dir)
@@ -80,6 +81,7 @@ def build_model(model_dir: str | Path, dtype: torch.dtype, device: str | torch.d
         init_random_weights(model, seed)
     else:
         load_weights(model, model_dir, strict=strict)
+    model.pack_product_weights(pack_weights)
     return model
 
 

@@ -162,6 +162,40 @@ class DecoderModel:
     def num_param_bytes(self) -> int:
         return sum(bp.tensor.numel() * bp.tensor.element_size() for bp in self.params.values())
 
+    # ------------------------------------------------------------------ packed copies
+    def product_weights(self) -> list[torch.Tensor]:
+        """The matrices that the parts stream in decode steps and that can be packed, each once
+        (a tied head names the embedding's)."""
+        seen: dict[int, torch.Tensor] = {}
+        for _, part in self._owned:
+            for name in part.product_weights():
+                t = part.params.get(name)
+                if t is not None and ops.can_pack_weight(t):
+                    seen.setdefault(id(t), t)
+        return list(seen.values())
+
+    def pack_product_weights(self, enable: bool | None = None) -> int:
+        """Give every such matrix its packed twin (``ops.pack_weight``); returns the bytes
+        taken.  ``enable`` None decides by room: the copies are made if they fit in a quarter
+        of the device's memory and leave half of what is free now (a model that fills the
+        device keeps its matrices as they are).  Call again after the weights changed."""
+        if self.device.type != "cuda" or self.dtype != torch.bfloat16:
+            return 0
+        weights = self.product_weights()
+        need = sum(w.numel() * w.element_size() for w in weights)
+        if enable is None:
+            free, total = torch.cuda.mem_get_info(self.device)
+            already = sum(w.kvc_packed.numel() * 2 for w in weights if getattr(w, "kvc_packed", None) is not None)
+            enable = need <= total // 4 and need - already <= free // 2
+        if not enable:
+            for w in weights:
+                if hasattr(w, "kvc_packed"):
+                    del w.kvc_packed
+            return 0
+        for w in weights:
+            ops.pack_weight(w)
+        return need
+
     # ----------------------------------------------------------------------- forward
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """Normalised hidden rows ``[T, H]`` in the model dtype for the batch in ``ctx``."""

@@ -54,10 +54,11 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_gemm_mid_slices": [I, I],
         "kvc_gemm_mid_bf16": [P, P, P, P, P, I, I, I, L, L, I, I, P],
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
-        "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, P],
-        "kvc_gemm_skinny_silu_mul_bf16": [P, P, P, P, I, I, I, L, L, P],
+        "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, I, P],
+        "kvc_gemm_skinny_silu_mul_bf16": [P, P, P, P, I, I, I, L, L, I, P],
+        "kvc_pack_weight": [P, P, I, I, P],
         "kvc_gemm_skinny_blocks": [I, I, I],
-        "kvc_gemm_skinny_fused_bf16": [P, P, P, P, I, I, I, L, L, I, P, I, I, F, P, L, P, P, P],
+        "kvc_gemm_skinny_fused_bf16": [P, P, P, P, I, I, I, L, L, I, P, I, I, F, P, L, P, P, I, P],
         "kvc_table_update": [P, I, I, P, I, P],
         "kvc_argmax": [P, P, I, I, L, P, P, I, P],
         "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P, L, I, P],
@@ -410,6 +411,38 @@ SKINNY_MAX_ROWS = 64
 SKINNY_PREFERRED_ROWS = 16
 
 
+def can_pack_weight(w: torch.Tensor) -> bool:
+    return (w.dim() == 2 and w.dtype == torch.bfloat16 and w.is_cuda and w.is_contiguous()
+            and w.shape[0] % 16 == 0 and w.shape[1] % 64 == 0)
+
+
+def pack_weight(w: torch.Tensor) -> torch.Tensor:
+    """A copy of the bfloat16 matrix ``w [N, K]`` in tiles of 16 rows x 32 columns, each 1 KB in
+    one piece, the tiles of 16 rows one after the other along K: the order in which the
+    weight-streaming products for few rows read a matrix, so that a load of theirs is one
+    contiguous kilobyte instead of 64 bytes from each of 16 rows (some 8% more bandwidth on
+    this chip).  The copy is kept as ``w.kvc_packed``; the products find it there and give
+    the same bits with it as without."""
+    if not can_pack_weight(w):
+        raise KernelError("pack_weight: a contiguous bfloat16 GPU matrix of a multiple of 16 rows "
+                          "and a multiple of 64 columns")
+    packed = torch.empty_like(w)
+    _check(load().kvc_pack_weight(packed.data_ptr(), w.data_ptr(), w.shape[0], w.shape[1], _stream()),
+           "kvc_pack_weight")
+    w.kvc_packed = packed
+    return packed
+
+
+def _streamed(w: torch.Tensor, rows: int | None = None) -> tuple[int, int]:
+    """(pointer, packed flag) of the matrix a weight-streaming product should read: the packed
+    twin of ``w`` where there is one (``rows``: the product's own row count, a multiple of 16
+    for a packed matrix, which the gated product's half must be too)."""
+    packed = getattr(w, "kvc_packed", None)
+    if packed is not None and (rows is None or rows % 16 == 0):
+        return packed.data_ptr(), 1
+    return _dev(w, "w"), 0
+
+
 def gemm_skinny_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor,
                      bias: torch.Tensor | None = None) -> None:
     """``out = a @ w.T (+ bias)`` for up to 64 rows of bfloat16; ``out`` is bfloat16 or
@@ -422,9 +455,10 @@ def gemm_skinny_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor,
         raise KernelError("gemm_skinny_bf16: operands must be bfloat16 GPU tensors")
     if bias is not None and (bias.dtype != torch.bfloat16 or bias.shape != (N,)):
         raise KernelError("gemm_skinny_bf16: bias must be bfloat16 [N]")
-    _check(load().kvc_gemm_skinny_bf16(out.data_ptr(), a.data_ptr(), _dev(w, "w"),
+    w_ptr, packed = _streamed(w)
+    _check(load().kvc_gemm_skinny_bf16(out.data_ptr(), a.data_ptr(), w_ptr,
                                        None if bias is None else _dev(bias, "bias"), M, N, K,
-                                       a.stride(0), out.stride(0), _code(out, "out"), _stream()),
+                                       a.stride(0), out.stride(0), _code(out, "out"), packed, _stream()),
            "kvc_gemm_skinny_bf16")
 
 
@@ -545,10 +579,11 @@ def _fused_skinny(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows
         residual = gain = out_ss = None
         ldr = 0
     if M:
+        w_ptr, packed = _streamed(w, N)
         _check(load().kvc_gemm_skinny_fused_bf16(
-            c_ptr, data.data_ptr(), _dev(w, "w"), None if bias is None else _dev(bias, "bias"), M, N, K,
+            c_ptr, data.data_ptr(), w_ptr, None if bias is None else _dev(bias, "bias"), M, N, K,
             data.stride(0), ldc, int(gated), in_ss or None, in_parts, in_width, float(in_eps),
-            residual, ldr, gain, out_ss, _stream()), "kvc_gemm_skinny_fused_bf16")
+            residual, ldr, gain, out_ss, packed, _stream()), "kvc_gemm_skinny_fused_bf16")
     return result
 
 
@@ -667,9 +702,10 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
             return
         if bias is not None and (bias.dtype != torch.bfloat16 or bias.shape != (2 * I,)):
             raise KernelError("linear_silu_mul: bias must be bfloat16 [2I]")
+        w_ptr, packed = _streamed(w, I)
         _check(load().kvc_gemm_skinny_silu_mul_bf16(
-            out.data_ptr(), x.data_ptr(), _dev(w, "w"), None if bias is None else _dev(bias, "bias"),
-            M, I, K, x.stride(0), out.stride(0), _stream()), "kvc_gemm_skinny_silu_mul_bf16")
+            out.data_ptr(), x.data_ptr(), w_ptr, None if bias is None else _dev(bias, "bias"),
+            M, I, K, x.stride(0), out.stride(0), packed, _stream()), "kvc_gemm_skinny_silu_mul_bf16")
         return
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and x.is_cuda and FOLD_ROWS < M <= MID_ROWS and mid_operands_ok(x, w)

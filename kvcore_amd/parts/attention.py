@@ -128,6 +128,9 @@ class PagedAttention(Mixer):
     def cache_need(self) -> CacheNeed:
         return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
 
+    def product_weights(self) -> tuple[str, ...]:
+        return ("qkv_proj.weight", "o_proj.weight")
+
     def forward(self, x, ctx, call, sink=None):
         p = self.params
         qkv = ctx.buf("attn_qkv", self.q_size + 2 * self.kv_size)

@@ -96,6 +96,12 @@ class Part:
     def param_specs(self) -> list[ParamSpec]:
         return []
 
+    def product_weights(self) -> tuple[str, ...]:
+        """Local names of the parameters that this part hands to ``ops.linear`` and its
+        kin as weight matrices: the model may keep a second copy of them in the order in
+        which decode steps stream them (``ops.pack_weight``)."""
+        return ()
+
     def setup(self, runtime: Runtime) -> None:
         """Called once after construction, before parameters are bound."""
         self.runtime = runtime

@@ -38,6 +38,9 @@ class OutputHead(Part):
     def param_specs(self) -> list[ParamSpec]:
         return [] if self.tied else [ParamSpec("weight", (self.vocab_size, self.hidden_size))]
 
+    def product_weights(self) -> tuple[str, ...]:
+        return ("weight",)
+
     def forward(self, logits: torch.Tensor, hidden_rows: torch.Tensor, ctx) -> None:
         """``logits [S, V]`` float32 from ``hidden_rows [S, H]`` in the model dtype."""
         w = self.params["weight"]

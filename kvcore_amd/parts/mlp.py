@@ -42,6 +42,9 @@ class SwiGLU(FeedForward):
             specs.append(ParamSpec("down_proj.bias", (H,), init="zeros"))
         return specs
 
+    def product_weights(self) -> tuple[str, ...]:
+        return ("gate_up_proj.weight", "down_proj.weight")
+
     def forward(self, x, ctx, call, sink=None):
         p = self.params
         act = ctx.buf("ffn_act", self.intermediate_size)

@@ -492,3 +492,29 @@ def test_random_configurations(tmp_path, seed):
         assert len(got) == sum(len(t) for t in token_lists.values())
         compare(got, expect, dtype, logit_rms=rms)
         assert session.manager.num_free_pages()[0] == session.num_pages - 1
+
+
+def test_packed_weights_change_no_bit(models):
+    """A model keeps a second copy of its matrices in the order decode steps stream them
+    (where the device has room, so in every other test here).  The logits with it are those
+    without it, bit for bit: whole prompt, then tokens one by one."""
+    from kvcore_amd.engine.replay import TraceSession
+    from kvcore_amd.engine.runner import build_model
+
+    folder, cfg, weights, page = models["D"]
+    tokens = random_tokens(90, cfg["vocab_size"], seed=77)
+    rows = {}
+    for pack in (True, False):
+        model = build_model(folder, torch.bfloat16, "cuda:0", pack_weights=pack)
+        packed = [w for w in model.product_weights() if getattr(w, "kvc_packed", None) is not None]
+        assert len(packed) == (len(model.product_weights()) if pack else 0)
+        assert not pack or len(packed) >= 4 * cfg["num_hidden_layers"] + 1
+        session = TraceSession(str(folder), torch.bfloat16, max_tokens=128, block_size=page, model=model)
+        steps = [{"step": 0, "entries": [{"id": "r", "tokens": tokens[:60], "want": [59]}], "end": []}]
+        steps += [{"step": i + 1, "entries": [{"id": "r", "tokens": [tokens[60 + i]], "want": [0]}], "end": []}
+                  for i in range(30)]
+        rows[pack] = collect(session, steps)
+    assert len(rows[True]) == 31
+    for key, row in rows[True].items():
+        assert torch.equal(row, rows[False][key]), key
+    compare(rows[True], {"r": oracle("D", cfg, weights, tokens)}, torch.bfloat16)

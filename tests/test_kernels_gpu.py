@@ -296,6 +296,55 @@ def test_linear_silu_mul(ops, M, I, K, with_bias):
     assert torch.allclose(out.double(), want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 16, 64), (3, 64, 128), (8, 4096, 4096), (8, 144, 1088), (16, 1024, 512),
+                                   (40, 96, 192)])
+def test_packed_weights_give_the_same_bits(ops, M, N, K):
+    """``pack_weight`` stores the matrix in the order the few-row products read it; they must
+    give, bit for bit, what they give from the plain matrix: plain, gated, with the norms
+    folded in, with bias."""
+    x = rnd(M, K, dtype=torch.bfloat16, seed=1)
+    w = (rnd(N, K, dtype=torch.bfloat16, seed=2) * 0.1).contiguous()
+    bias = rnd(N, dtype=torch.bfloat16, seed=3)
+    ss = (rnd(M, 4, seed=5).abs() + 0.5).contiguous()
+    gain = rnd(N, seed=6).abs() + 0.5
+    plain_out = {}
+    for packed in (False, True):
+        if packed:
+            tiles = ops.pack_weight(w)
+            # element (n, k) sits at ((n / 16) * (K / 32) + k / 32) * 512 + (n % 16) * 32 + k % 32
+            want = w.view(N // 16, 16, K // 32, 32).permute(0, 2, 1, 3).contiguous().view(N, K)
+            assert torch.equal(tiles.view(torch.int16), want.view(torch.int16)) and w.kvc_packed is tiles
+        outs = []
+        for out_dtype in (torch.bfloat16, torch.float32):
+            out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+            ops.gemm_skinny_bf16(out, x, w, bias)
+            outs.append(out)
+        if N % 32 == 0:  # gated: the first half of the rows is the gate, the second the up factor
+            out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
+            ops.linear_silu_mul(out, x, w, bias, lambda: torch.empty(M, N, dtype=torch.bfloat16, device=DEV))
+            outs.append(out)
+        if M <= 16:
+            # the fold: scaled rows in, residual sink out
+            rows = ops.ScaledRows(x, ss, K, 1e-5)
+            residual = rnd(M, N, dtype=torch.float32, seed=4)
+            sink = ops.ResidualSink(residual=residual, gain=gain, eps=1e-5,
+                                    out=torch.empty(M, N, dtype=torch.bfloat16, device=DEV),
+                                    ss_parts=torch.empty(M * ops.skinny_blocks(N, K), device=DEV))
+            got = ops.linear(sink, rows, w, bias)
+            outs += [sink.out.clone(), residual.clone(), got.ss_parts.clone()]
+        if packed:
+            assert len(outs) == len(plain_out["outs"])
+            for a, b in zip(outs, plain_out["outs"]):
+                assert torch.equal(a.view(torch.int16 if a.dtype == torch.bfloat16 else torch.int32),
+                                   b.view(torch.int16 if b.dtype == torch.bfloat16 else torch.int32))
+        else:
+            plain_out["outs"] = outs
+    ref = x.float() @ w.float().t() + bias.float()
+    assert torch.allclose(plain_out["outs"][1], ref, atol=2e-2, rtol=2e-2)
+    with pytest.raises(ops.KernelError, match="pack_weight"):
+        ops.pack_weight(w[:, :32])
+
+
 def test_linear_picks_a_kernel_by_row_count(ops):
     w = rnd(96, 256, dtype=torch.bfloat16, seed=5, scale=0.05)
     for M in (3, 64, 65, 200):
