@@ -42,7 +42,7 @@ template <int WAVES, int RT, int NT, bool GATED, typename OutT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_mid_kernel(
     OutT* __restrict__ C, float* __restrict__ partial, const bf16_t* __restrict__ A,
     const bf16_t* __restrict__ W, const bf16_t* __restrict__ bias, int M, int N, int K, int64_t lda,
-    int64_t ldc, int k_per_block) {
+    int64_t ldc, int k_per_block, int packed) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
   static_assert(kStages % (2 * kChunkSteps) == 0, "a round of stages must cover whole pairs of chunks");
   __shared__ __attribute__((aligned(16))) bf16_t a_lds[2][NT * 16 * kRowElems];
@@ -62,12 +62,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mid_kernel(
   const int k_end = (k_begin + k_per_block < K) ? k_begin + k_per_block : K;
   const int n_steps = (k_end - k_begin) / 64;  // the host makes slices whole rounds of steps
 
+  const int ks = packed ? 16 : 1;
   const bf16_t* wp[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const int r = GATED ? n0 + col : n0 + rt * 16 + col;
     const int64_t row = (r < N ? r : N - 1) + ((GATED && rt == 1) ? N : 0);
-    wp[rt] = W + row * K + k_begin + 8 * quad;
+    // packed: what kvc_pack_weight made of W (tiles of 16 rows x 32 k, 1 KB each, along K)
+    wp[rt] = packed ? W + (row >> 4) * (static_cast<int64_t>(K) * 16) + (row & 15) * 32 +
+                          static_cast<int64_t>(k_begin) * 16 + 8 * quad
+                    : W + row * K + k_begin + 8 * quad;
   }
   // this thread's pieces of a chunk of A: rows beyond M read the last row and are dropped
   // at the end
@@ -101,8 +105,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mid_kernel(
     const int k = 64 * where(step);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      wbuf[stage][rt][0] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k);
-      wbuf[stage][rt][1] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k + 32);
+      wbuf[stage][rt][0] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + k * ks);
+      wbuf[stage][rt][1] = *reinterpret_cast<const bf16x8_t*>(wp[rt] + (k + 32) * ks);
     }
   };
   auto fetch_chunk = [&](int slot, int chunk) {
@@ -254,6 +258,7 @@ struct MidPlan {
   int rt;      // 16-row tiles per wave
   int slices;  // along K
   int k_per_block;
+  int packed;  // W is in kvc_pack_weight's order
 };
 
 // Blocks enough for every compute unit, from N and K alone.  Narrow outputs are cut along K
@@ -261,6 +266,7 @@ struct MidPlan {
 // KVC_MID_WAVES / KVC_MID_RT / KVC_MID_SLICES override the choice for tuning.
 MidPlan plan_mid(int N, int K, bool gated, bool may_slice) {
   MidPlan p;
+  p.packed = 0;
   // two waves a block where four would leave compute units without one
   p.waves = (gated && (N + 63) / 64 < 192) ? 2 : 4;
   p.rt = gated ? 2 : (N >= 16384 ? 2 : 1);
@@ -293,7 +299,7 @@ void launch_mid(OutT* C, float* partial, const bf16_t* A, const bf16_t* W, const
   const int cols_per_block = WAVES * (GATED ? 16 : 16 * RT);
   const dim3 grid((N + cols_per_block - 1) / cols_per_block, p.slices), block(WAVES * 64);
   hipLaunchKernelGGL((gemm_mid_kernel<WAVES, RT, NT, GATED, OutT>), grid, block, 0, stream, C,
-                     p.slices > 1 ? partial : nullptr, A, W, bias, M, N, K, lda, ldc, p.k_per_block);
+                     p.slices > 1 ? partial : nullptr, A, W, bias, M, N, K, lda, ldc, p.k_per_block, p.packed);
 }
 
 template <bool GATED, typename OutT>
@@ -346,8 +352,9 @@ extern "C" int kvc_gemm_mid_slices(int N, int K) {
 
 extern "C" int kvc_gemm_mid_bf16(void* C, void* partial, const void* A, const void* W, const void* bias,
                                  int M, int N, int K, int64_t lda, int64_t ldc, int out_dtype, int mode,
-                                 kvc_stream stream) {
+                                 int packed, kvc_stream stream) {
   if (int rc = check_mid(A, W, M, N, K, lda, ldc)) return rc;
+  if (packed && N % 16) return kvc_fail("kvc_gemm_mid_bf16: packed weights have a multiple of 16 rows");
   if (mode < 0 || mode > 3) return kvc_fail("kvc_gemm_mid_bf16: unknown mode");
   if (M == 0) return 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -357,12 +364,14 @@ extern "C" int kvc_gemm_mid_bf16(void* C, void* partial, const void* A, const vo
   float* part = static_cast<float*>(partial);
   if (mode == 1) {  // silu(A Wg^T) * (A Wu^T): one slice, bfloat16
     if (out_dtype != 1) return kvc_fail("kvc_gemm_mid_bf16: the gated form stores bfloat16");
-    return dispatch_mid<true>(static_cast<bf16_t*>(C), nullptr, a, w, b, M, N, K, lda, ldc,
-                              plan_mid(N, K, true, false), s);
+    MidPlan p = plan_mid(N, K, true, false);
+    p.packed = packed;
+    return dispatch_mid<true>(static_cast<bf16_t*>(C), nullptr, a, w, b, M, N, K, lda, ldc, p, s);
   }
   if (mode == 2) {  // only the slices' partial sums
     if (part == nullptr) return kvc_fail("kvc_gemm_mid_bf16: the partial sums need their buffer");
     MidPlan p = plan_mid(N, K, false, true);
+    p.packed = packed;
     if (p.slices == 1) {  // a single slice is the result: float32 [M, N]
       return dispatch_mid<false>(part, nullptr, a, w, nullptr, M, N, K, lda, N, p, s);
     }
@@ -370,6 +379,7 @@ extern "C" int kvc_gemm_mid_bf16(void* C, void* partial, const void* A, const vo
   }
   // plain product: one slice at once, or (mode 3, given a buffer) slices and their sum
   MidPlan p = plan_mid(N, K, false, mode == 3 && part != nullptr);
+  p.packed = packed;
   if (out_dtype != 0 && out_dtype != 1) return kvc_fail("kvc_gemm_mid_bf16: unknown output dtype code");
   if (p.slices == 1) {
     if (out_dtype == 0)

@@ -135,10 +135,11 @@ int kvc_gemm_f32(float* C, const float* A, const float* W, const float* bias, in
 // then Wu.  mode 2: narrow outputs are cut along K into kvc_gemm_mid_slices(N, K) slices and
 // only their float32 partial sums are stored, partial [slices, M, N] (no bias); the kernel
 // that consumes them adds them up in slice order.  mode 3: as mode 0, but cut along K like
-// mode 2 when `partial` is given, with a second kernel that sums the slices.
+// mode 2 when `partial` is given, with a second kernel that sums the slices.  With `packed` W
+// is what kvc_pack_weight made of the matrix (the same sums, read in contiguous kilobytes).
 int kvc_gemm_mid_slices(int N, int K);
 int kvc_gemm_mid_bf16(void* C, void* partial, const void* A, const void* W, const void* bias, int M,
-                      int N, int K, int64_t lda, int64_t ldc, int out_dtype, int mode,
+                      int N, int K, int64_t lda, int64_t ldc, int out_dtype, int mode, int packed,
                       kvc_stream stream);
 
 // C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) for M <= 64 rows of bfloat16 on the matrix

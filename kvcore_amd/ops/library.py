@@ -52,7 +52,7 @@ def _declare(lib: ctypes.CDLL) -> None:
                                   P, P, I, I, P],
         "kvc_prefill_attention_supported": [I, I, I, I, I],
         "kvc_gemm_mid_slices": [I, I],
-        "kvc_gemm_mid_bf16": [P, P, P, P, P, I, I, I, L, L, I, I, P],
+        "kvc_gemm_mid_bf16": [P, P, P, P, P, I, I, I, L, L, I, I, I, P],
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
         "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, I, P],
         "kvc_gemm_skinny_silu_mul_bf16": [P, P, P, P, I, I, I, L, L, I, P],
@@ -632,9 +632,10 @@ def gemm_mid(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias: t
         if partial.dtype != torch.float32 or partial.numel() < mid_slices(N, K) * M * N:
             raise KernelError("gemm_mid: the buffer for partial sums is too small")
         part_ptr = _dev(partial, "partial", torch.float32)
-    _check(load().kvc_gemm_mid_bf16(out_ptr, part_ptr, x.data_ptr(), _dev(w, "w"),
+    w_ptr, packed = _streamed(w, N)
+    _check(load().kvc_gemm_mid_bf16(out_ptr, part_ptr, x.data_ptr(), w_ptr,
                                     None if bias is None else _dev(bias, "bias"), M, N, K, x.stride(0),
-                                    ldc, code, mode, _stream()), "kvc_gemm_mid_bf16")
+                                    ldc, code, mode, packed, _stream()), "kvc_gemm_mid_bf16")
 
 
 def add_slices_rmsnorm(out: torch.Tensor, residual: torch.Tensor, partial: torch.Tensor, slices: int,

@@ -345,6 +345,36 @@ def test_packed_weights_give_the_same_bits(ops, M, N, K):
         ops.pack_weight(w[:, :32])
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 64, 512), (40, 1008, 1024), (64, 4096, 1536)])
+def test_packed_weights_give_the_same_bits_at_a_few_dozen_rows(ops, M, N, K):
+    x = rnd(M, K, dtype=torch.bfloat16, seed=1)
+    w = (rnd(N, K, dtype=torch.bfloat16, seed=2) * 0.1).contiguous()
+    bias = rnd(N, dtype=torch.bfloat16, seed=3)
+    results = []
+    for packed in (False, True):
+        if packed:
+            ops.pack_weight(w)
+        outs = []
+        for mode in (0, 3):
+            for out_dtype in (torch.bfloat16, torch.float32):
+                out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+                part = torch.empty(ops.mid_slices(N, K) * M * N, device=DEV)
+                ops.gemm_mid(out, x, w, bias, mode=mode, partial=part if mode == 3 else None)
+                outs.append(out)
+        part = torch.zeros(ops.mid_slices(N, K) * M * N, device=DEV)
+        ops.gemm_mid(None, x, w, mode=2, partial=part)
+        outs.append(part)
+        if N % 32 == 0:
+            out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
+            ops.gemm_mid(out, x, w, bias, mode=1)
+            outs.append(out)
+        results.append(outs)
+    for a, b in zip(*results):
+        bits = torch.int16 if a.dtype == torch.bfloat16 else torch.int32
+        assert torch.equal(a.view(bits), b.view(bits))
+    assert torch.allclose(results[0][1], x.float() @ w.float().t() + bias.float(), atol=3e-2, rtol=2e-2)
+
+
 def test_linear_picks_a_kernel_by_row_count(ops):
     w = rnd(96, 256, dtype=torch.bfloat16, seed=5, scale=0.05)
     for M in (3, 64, 65, 200):
