@@ -249,8 +249,9 @@ class EngineCore:
         in flight, each request's token being read from where that one's sampling leaves it.
         The host's work for a step then overlaps the device's work for the step before.  A
         request that turns out to have ended on a stop token has run one token too many,
-        which is dropped (``_keep_in_flight``); its keys and values went to pages that
-        were still its own."""
+        which is dropped (``_keep_in_flight``).  Its key and value land in a page that the
+        host has given back by then; on the device that write comes before anything a later
+        owner of the page does, and an owner reads only the slots it has written itself."""
         if flight.row_ids != [s.request_id for s in flight.output.scheduled]:
             return None  # a request was dropped from it: its rows are not the next step's rows
         planned = self.scheduler.plan_decode_ahead(flight.output)
