@@ -418,9 +418,12 @@ void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M
 // how many rows come with it.  Measured on MI355X at 1 to 16 rows: 4 waves along K; outputs
 // wider than 4096 want 32 weight rows a wave, narrower ones 16.
 // KVC_SKINNY_RT / KVC_SKINNY_WAVES override the choice for tuning.
-inline void pick_shape(int N, int K, int* rt_out, int* waves_out) {
+// From a packed matrix a wave takes 16 rows whatever N is: its second 16 rows would be a
+// second stream 16 * K elements behind the first, and the two together read slower than one
+// (128256 x 4096: 199 against 172 us; 28672 x 4096: 50.5 against 40.6 us).
+inline void pick_shape(int N, int K, int packed, int* rt_out, int* waves_out) {
   int rt, waves;
-  if (N > 4096) {
+  if (N > 4096 && !packed) {
     rt = 2;
     waves = 4;
   } else {
@@ -442,7 +445,7 @@ template <typename OutT>
 int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N, int K,
              int64_t lda, int64_t ldc, const SkinnyExtras& ex, int packed, hipStream_t stream) {
   int rt, waves;
-  pick_shape(N, K, &rt, &waves);
+  pick_shape(N, K, packed, &rt, &waves);
   const int nt = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 63) / 64 * 64;
@@ -566,11 +569,11 @@ extern "C" int kvc_pack_weight(void* dst, const void* src, int N, int K, kvc_str
   return kvc_check_launch("kvc_pack_weight");
 }
 
-extern "C" int kvc_gemm_skinny_blocks(int N, int K, int gated) {
+extern "C" int kvc_gemm_skinny_blocks(int N, int K, int gated, int packed) {
   if (N <= 0 || K <= 0) return 0;
   if (gated) return (N + 15) / 16;
   int rt, waves;
-  pick_shape(N, K, &rt, &waves);
+  pick_shape(N, K, packed, &rt, &waves);
   return (N + 16 * rt - 1) / (16 * rt);
 }
 

@@ -173,10 +173,10 @@ int kvc_gemm_skinny_silu_mul_bf16(void* C, const void* A, const void* W, const v
 //    before bias (and activation);
 //  - residual [M, ldr] float32 (or null; not with gated): residual += product (+ bias); C
 //    receives bfloat16(residual * gain[n]) and out_ss [M, blocks] the new residual's sums of
-//    squares per block of columns, blocks = kvc_gemm_skinny_blocks(N, K, 0): the in_ss of the
+//    squares per block of columns, blocks = kvc_gemm_skinny_blocks(N, K, 0, packed): the in_ss of the
 //    product that consumes C.
 // gated = 1 is kvc_gemm_skinny_silu_mul_bf16's product (N = the gate's rows).
-int kvc_gemm_skinny_blocks(int N, int K, int gated);
+int kvc_gemm_skinny_blocks(int N, int K, int gated, int packed);
 int kvc_gemm_skinny_fused_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
                                int K, int64_t lda, int64_t ldc, int gated, const float* in_ss,
                                int in_parts, int in_width, float in_eps, float* residual,

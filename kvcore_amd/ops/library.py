@@ -57,7 +57,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, I, P],
         "kvc_gemm_skinny_silu_mul_bf16": [P, P, P, P, I, I, I, L, L, I, P],
         "kvc_pack_weight": [P, P, I, I, P],
-        "kvc_gemm_skinny_blocks": [I, I, I],
+        "kvc_gemm_skinny_blocks": [I, I, I, I],
         "kvc_gemm_skinny_fused_bf16": [P, P, P, P, I, I, I, L, L, I, P, I, I, F, P, L, P, P, I, P],
         "kvc_table_update": [P, I, I, P, I, P],
         "kvc_argmax": [P, P, I, I, L, P, P, I, P],
@@ -531,9 +531,9 @@ def rows_sinkable(num_rows: int, dtype: torch.dtype, width: int = 0) -> bool:
     return dtype == torch.bfloat16 and not rows_fusable(num_rows, dtype, width) and 0 < num_rows <= MID_ROWS
 
 
-def skinny_blocks(N: int, K: int, gated: bool = False) -> int:
+def skinny_blocks(N: int, K: int, gated: bool = False, packed: bool = False) -> int:
     """How many blocks of columns the weight-streaming kernel cuts ``N`` outputs into."""
-    return int(load().kvc_gemm_skinny_blocks(N, K, int(gated)))
+    return int(load().kvc_gemm_skinny_blocks(N, K, int(gated), int(packed)))
 
 
 def _fused_skinny(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: torch.Tensor,
@@ -557,7 +557,7 @@ def _fused_skinny(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows
         in_ss, in_width, in_eps = x.ss_parts.data_ptr(), x.width, x.eps
     result = None
     if isinstance(out, ResidualSink):
-        parts = skinny_blocks(N, K)
+        parts = skinny_blocks(N, K, packed=bool(_streamed(w, N)[1]))
         if out.residual.shape != (M, N) or out.residual.dtype != torch.float32 or out.residual.stride(1) != 1:
             raise KernelError("fused product: the residual must be float32 [T, N]")
         if out.gain.shape != (N,) or out.gain.dtype != torch.float32:
