@@ -82,8 +82,8 @@ class EngineCore:
                                 seed=config.load_config.seed, strict=config.load_config.strict,
                                 pack_weights=config.load_config.pack_decode_weights)
         self.model = model
-        logger.info("model ready in %.2f s (%d parameter bytes)", time.perf_counter() - t0,
-                    model.num_param_bytes())
+        logger.info("model ready in %.2f s (%d parameter bytes, %d more in packed copies)",
+                    time.perf_counter() - t0, model.num_param_bytes(), getattr(model, "packed_bytes", 0))
 
         sched = config.scheduler_config
         cache = config.cache_config

@@ -81,7 +81,7 @@ def build_model(model_dir: str | Path, dtype: torch.dtype, device: str | torch.d
         init_random_weights(model, seed)
     else:
         load_weights(model, model_dir, strict=strict)
-    model.pack_product_weights(pack_weights)
+    model.packed_bytes = model.pack_product_weights(pack_weights)
     return model
 
 
