@@ -193,6 +193,21 @@ int kvc_table_update(int32_t* table, int table_stride, int table_rows, const int
 int kvc_argmax(int32_t* out, const float* logits, int S, int V, int64_t row_stride,
                float* part_val, int32_t* part_idx, int part_capacity, kvc_stream stream);
 
+// kvc_argmax for callers that cannot allocate device memory and bring no workspace (code
+// under HIP graph capture, tight serving loops, harnesses that forbid allocation).  It has no
+// counterpart in the reference.  The partial results of long rows live in a static device
+// array of kvc_argmax_static_capacity() = 16384 entries (128 KB that every GPU the library
+// runs on holds until the process ends); S * ceil(V / 8192) beyond that is refused with an
+// error, rows of at most 8192 values need no partial results and are never refused.  The call
+// allocates and frees nothing, on the device or through any library.  The array keeps the last
+// call's contents; nothing in it has to start at zero, since every entry that is read was
+// written earlier in the same call.  All calls on one GPU share that GPU's array: calls that
+// overlap there (different streams or threads) race, calls on one stream do not.  The results
+// equal kvc_argmax's.
+int kvc_argmax_static_capacity(void);
+int kvc_argmax_static(int32_t* out, const float* logits, int S, int V, int64_t row_stride,
+                      kvc_stream stream);
+
 // Per row s: temperature[s] < 1e-5 gives the argmax; otherwise
 // argmax_v(logits[v] / temperature - log(e_v)), e_v exponential noise keyed by
 // (seed_lo[s], seed_hi[s], index[s], v), over the entries that top_k[s] (<= 0: all) and

@@ -11,6 +11,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "device_utils.h"
 #include "kvcore_hip.h"
 
@@ -600,6 +602,40 @@ __global__ void split_final_kernel(int32_t* __restrict__ out, const u64* __restr
   out[s] = packed ? static_cast<int32_t>(0xFFFFFFFFu - static_cast<uint32_t>(packed)) : 0;
 }
 
+// ------------------------------------------------------- argmax without a workspace argument
+// Partial results of the two-stage argmax for callers that can neither allocate nor bring a
+// workspace.  Every GPU that the library runs on holds its own copy of this array until the
+// process ends (128 KB).  In host code the array's name is a stand-in, not a device address:
+// only the pointer that hipGetSymbolAddress returns for the current device is passed on.
+// All calls on one GPU share that GPU's copy, so calls that overlap there (two streams, two
+// threads) race; calls on one stream follow each other and do not.
+constexpr int kStaticArgmaxEntries = 16384;
+constexpr int kStaticArgmaxDevices = 64;
+// values in the first half (float32), indices in the second (int32)
+static __device__ __align__(256) uint32_t scratch[2 * kStaticArgmaxEntries];
+
+uint32_t* g_static_scratch[kStaticArgmaxDevices];  // per device: its copy's address, once known
+std::mutex g_static_scratch_mutex;
+
+// The current device's copy of `scratch`, looked up once per device with that device current.
+int static_scratch_pointer(uint32_t** out) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kStaticArgmaxDevices)
+    return kvc_fail("kvc_argmax_static: cannot tell the current device");
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  if (g_static_scratch[device] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      return kvc_fail("kvc_argmax_static: hipGetSymbolAddress failed for the scratch array");
+    }
+    g_static_scratch[device] = static_cast<uint32_t*>(ptr);
+  }
+  *out = g_static_scratch[device];
+  return 0;
+}
+
 }  // namespace
 
 extern "C" int kvc_argmax(int32_t* out, const float* logits, int S_, int V, int64_t row_stride,
@@ -621,6 +657,36 @@ extern "C" int kvc_argmax(int32_t* out, const float* logits, int S_, int V, int6
   hipLaunchKernelGGL(argmax_kernel, dim3(S_), dim3(kThreads), 0,
                      reinterpret_cast<hipStream_t>(stream), out, logits, V, row_stride);
   return kvc_check_launch("kvc_argmax");
+}
+
+extern "C" int kvc_argmax_static_capacity(void) { return kStaticArgmaxEntries; }
+
+extern "C" int kvc_argmax_static(int32_t* out, const float* logits, int S_, int V,
+                                 int64_t row_stride, kvc_stream stream) {
+  if (S_ < 0 || V <= 0 || row_stride < V) return kvc_fail("kvc_argmax_static: bad sizes");
+  if (out == nullptr || logits == nullptr) return kvc_fail("kvc_argmax_static: null pointer");
+  if (S_ == 0) return 0;
+  constexpr int kChunk = 8192;
+  const int chunks = (V + kChunk - 1) / kChunk;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (chunks == 1) {  // a short row is one block's work and needs no partial results
+    hipLaunchKernelGGL(argmax_kernel, dim3(S_), dim3(kThreads), 0, st, out, logits, V, row_stride);
+    return kvc_check_launch("kvc_argmax_static");
+  }
+  if (chunks > 65535 || static_cast<int64_t>(S_) * chunks > kStaticArgmaxEntries)
+    return kvc_fail("kvc_argmax_static: rows x ceil(V / 8192) exceeds the 16384 partial results "
+                    "that the static scratch array holds; use kvc_argmax with a workspace");
+  uint32_t* ptr = nullptr;
+  if (static_scratch_pointer(&ptr) != 0) return -1;
+  float* part_val = reinterpret_cast<float*>(ptr);
+  int32_t* part_idx = reinterpret_cast<int32_t*>(ptr + kStaticArgmaxEntries);
+  // every partial result that stage two reads was written by stage one of this call, so the
+  // array's old contents need no clearing
+  hipLaunchKernelGGL(argmax_chunk_kernel, dim3(S_, chunks), dim3(kThreads), 0, st, part_val,
+                     part_idx, logits, V, row_stride, kChunk);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(S_), dim3(kWave), 0, st, out, part_val, part_idx,
+                     chunks);
+  return kvc_check_launch("kvc_argmax_static");
 }
 
 extern "C" int kvc_sample_workspace_words(int S_, int V) {

@@ -61,6 +61,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_gemm_skinny_fused_bf16": [P, P, P, P, I, I, I, L, L, I, P, I, I, F, P, L, P, P, I, P],
         "kvc_table_update": [P, I, I, P, I, P],
         "kvc_argmax": [P, P, I, I, L, P, P, I, P],
+        "kvc_argmax_static": [P, P, I, I, L, P],
         "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P, L, I, P],
         "kvc_sample_workspace_words": [I, I],
     }
@@ -71,6 +72,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.kvc_last_error.restype = ctypes.c_char_p
     lib.kvc_last_error.argtypes = []
     lib.kvc_version.restype = c_int
+    lib.kvc_argmax_static_capacity.restype = c_int
+    lib.kvc_argmax_static_capacity.argtypes = []
 
 
 def load(build_if_missing: bool = True) -> ctypes.CDLL:
