@@ -31,6 +31,22 @@ def cdiv(a: int, b: int) -> int:
     return -(-a // b)
 
 
+def plan_groups(needs, block_size: int, num_blocks: int) -> list[GroupConfig]:
+    """One ``GroupConfig`` per cache need (objects with ``page_size`` and ``window``, as
+    ``parts.base.CacheNeed``).  A group whose need names no page size has pages of
+    ``block_size`` tokens and ``num_blocks`` of them; a group with a page size of its own gets
+    as many pages as hold the same number of tokens.  Every count includes the null page."""
+    if num_blocks < 2:
+        raise ValueError(f"a cache needs the null page and at least one more, got {num_blocks}")
+    tokens = (num_blocks - 1) * block_size
+    out = []
+    for need in needs:
+        size = need.page_size or block_size
+        pages = num_blocks if size == block_size else cdiv(tokens, size) + 1
+        out.append(GroupConfig(size, pages, need.window))
+    return out
+
+
 @dataclass
 class _RequestPages:
     pages: list[int] = field(default_factory=list)  # entry i covers tokens [i*ps, (i+1)*ps)
@@ -39,7 +55,7 @@ class _RequestPages:
 
 class KVManager:
     def __init__(self, groups: list[GroupConfig], *, max_num_seqs: int, max_model_len: int,
-                 shuffle_seed: int | None = None) -> None:
+                 shuffle_seed: int | None = None, track_freed: bool = False) -> None:
         if max_model_len <= 0:
             raise ValueError("max_model_len must be positive")
         self.groups = list(groups)
@@ -49,6 +65,10 @@ class KVManager:
         self.max_model_len = max_model_len
         self._req_pages: dict[str, list[_RequestPages]] = {}
         self._req_slot: dict[str, int] = {}
+        # pages given back since the last ``drain_freed`` (a debugging aid: the runner may fill
+        # them with NaN; the reference keeps the like for new blocks, kv_manager.py:441-447)
+        self.track_freed = track_freed
+        self._freed: list[list[int]] = [[] for _ in self.groups]
 
     # ---------------------------------------------------------------------- admission
     def has_free_slot(self) -> bool:
@@ -112,12 +132,14 @@ class KVManager:
         ``num_computed - window + 1`` on; pages wholly before that are given back and
         read as the null page.  Returns per group how many leading entries are now null."""
         out = []
-        for g, pool, rp in zip(self.groups, self.pools, self._req_pages[request_id]):
+        for gi, (g, pool, rp) in enumerate(zip(self.groups, self.pools, self._req_pages[request_id])):
             if g.window > 0:
                 first_needed = max(num_computed - g.window + 1, 0)
                 upto = min(first_needed // g.page_size, len(rp.pages))
                 if upto > rp.released:
                     pool.give_back(rp.pages[rp.released:upto])
+                    if self.track_freed:
+                        self._freed[gi].extend(rp.pages[rp.released:upto])
                     for i in range(rp.released, upto):
                         rp.pages[i] = 0
                     rp.released = upto
@@ -136,9 +158,16 @@ class KVManager:
         pages are reused first (single_type_kv_manager.py:177-182), then the slot."""
         pages = self._req_pages.pop(request_id)
         slot = self._req_slot.pop(request_id)
-        for pool, rp in zip(self.pools, pages):
+        for gi, (pool, rp) in enumerate(zip(self.pools, pages)):
             pool.give_back(reversed(rp.pages))
+            if self.track_freed:
+                self._freed[gi].extend(p for p in rp.pages if p)
         self.slots.give_back(slot)
+
+    def drain_freed(self) -> list[list[int]]:
+        """Per group, the pages given back since the last call (empty without ``track_freed``)."""
+        out, self._freed = self._freed, [[] for _ in self.groups]
+        return out
 
     # --------------------------------------------------------------------- inspection
     def num_free_pages(self) -> list[int]:

@@ -77,12 +77,16 @@ class LoadConfig:
 @dataclass(frozen=True)
 class CacheConfig:
     """Reference: config.py:43-60.  ``num_gpu_blocks`` counts pages including the
-    reserved null page; when given it wins over profiling."""
+    reserved null page; when given it wins over profiling.  ``poison_pages`` is a debugging
+    aid of this engine: every page is filled with NaN when a request first gets it and when
+    it is given back, so that a read of a slot its request did not write shows in the logits
+    (the reference zeroes new blocks instead, kvcore/model/model_runner.py:646-657)."""
 
     block_size: int = 16
     num_gpu_blocks: int | None = None
     profile_kv_cache: bool = True
     gpu_memory_utilization: float = 0.9
+    poison_pages: bool = False
 
     def __post_init__(self) -> None:
         if self.block_size <= 0:

@@ -209,6 +209,25 @@ class LlamaConfig:
         return out
 
 
+def read_generation_eos(model_dir: str | Path) -> tuple[int, ...]:
+    """``eos_token_id`` (an int or a list) of ``<model_dir>/generation_config.json``; empty if
+    the file or the key is absent.  Instruct checkpoints of Llama 3 list their end-of-turn
+    id there and not in config.json."""
+    path = Path(model_dir).expanduser() / "generation_config.json"
+    if not path.is_file():
+        return ()
+    try:
+        data = json.loads(path.read_text())
+    except (OSError, ValueError) as exc:
+        raise ConfigError(f"{path}: not readable as JSON: {exc}") from exc
+    eos = data.get("eos_token_id") if isinstance(data, dict) else None
+    if eos is None:
+        return ()
+    if isinstance(eos, (list, tuple)):
+        return tuple(int(e) for e in eos)
+    return (int(eos),)
+
+
 def read_config_json(model_dir: str | Path) -> dict[str, Any]:
     """The raw mapping of ``<model_dir>/config.json``.  A missing folder raises
     ``FileNotFoundError`` as the reference does (model_loader/default_loader.py:98-102)."""

@@ -457,10 +457,11 @@ int launch_decode(DecodeArgs& args, int T, hipStream_t stream) {
   if (args.lds_pages > args.table_stride) args.lds_pages = args.table_stride;
   int waves = decode_waves(g, D);
   // more blocks than compute units: smaller blocks pack better
-  if (static_cast<int64_t>(T) * args.nkv * args.nsplit > 256 && waves > 4) waves = 4;
+  if (static_cast<int64_t>(T) * args.nkv * args.nsplit > kvc_device_compute_units() && waves > 4) waves = 4;
   while (waves > 1 && lds_total(waves, g, D, args.lds_pages) > kLdsLimit) waves /= 2;
   if (lds_total(waves, g, D, args.lds_pages) > kLdsLimit)
-    return kvc_fail("kvc_decode_attention: the block table is too wide for one split (use more)");
+    return kvc_fail("kvc_decode_attention: the block table is wider than kvc_decode_attention_max_table "
+                    "allows for one split");
   hipLaunchKernelGGL(decode_attention_kernel<D>, dim3(T, args.nkv, args.nsplit), dim3(waves * 64),
                      lds_total(waves, g, D, args.lds_pages), stream, args);
   if (args.nsplit > 1)
@@ -486,6 +487,14 @@ extern "C" int kvc_decode_attention_supported(int nh, int nkv, int d, int page_s
   if (nkv <= 0 || nh % nkv || nh / nkv > 16) return 0;
   if (page_size % 16) return 0;
   return d == 32 || d == 64 || d == 96 || d == 128 || d == 160 || d == 192 || d == 224 || d == 256;
+}
+
+extern "C" int kvc_decode_attention_max_table(int nh, int nkv, int d) {
+  if (nkv <= 0 || nh % nkv || d <= 0) return 0;
+  const size_t fixed = lds_total(1, nh / nkv, d, 0);
+  if (fixed >= kLdsLimit) return 0;
+  // launch_decode keeps two entries of slack beyond a split's share of the table
+  return static_cast<int>((kLdsLimit - fixed) / 4) - 2;
 }
 
 extern "C" int kvc_decode_attention_waves(int nh, int nkv, int d) {

@@ -611,29 +611,31 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
   const int64_t pairs1 = static_cast<int64_t>((tiles1 + 1) / 2) * nkv;
   const int64_t small_tiles = static_cast<int64_t>(tiles1) * nkv;
   const bool long_requests = T / R >= (D == 64 ? 512 : 1024);
+  // the thresholds below were measured on 256 compute units and are kept as multiples of them
+  const int cu = kvc_device_compute_units();
   int ct = 1, single = 0, waves = 4;
   if (g > 64) {
     ct = 2;
   } else if (nsplit > 1) {
     // very few rows: small tiles one a block reach the blocks wanted with a quarter of the
     // splits (128 rows at 1,024 keys: 21 against 39 us)
-    if (small_tiles <= 128) {
+    if (small_tiles <= cu / 2) {
       single = 1;
     } else {
       ct = 2;
       if (long_requests) waves = 8;  // 2,048 tokens after 30,000: 1.38 against 1.32 ms
     }
-  } else if (pairs1 > 512) {
+  } else if (pairs1 > 2 * cu) {
     ct = 2;
     if (long_requests) waves = 8;
-  } else if (pairs1 > 256) {
+  } else if (pairs1 > cu) {
     if (long_requests) {
       waves = 8;
-      single = pairs1 <= 448;
+      single = pairs1 <= 7 * cu / 4;
     }
   } else {
     single = 1;
-    if (D == 64 && pairs1 > 128 && long_requests) waves = 8;
+    if (D == 64 && pairs1 > cu / 2 && long_requests) waves = 8;
   }
   // KVC_PREFILL_MODE = 1p | 1s | 2p | 2s, then 4 or 8 (waves), overrides the choice for tuning
   static const char* mode = getenv("KVC_PREFILL_MODE");

@@ -95,3 +95,6 @@ __device__ __forceinline__ float block_sum(float v, float* scratch /* >= 16 floa
 // message that kvc_last_error() returns.
 int kvc_fail(const char* message);
 int kvc_check_launch(const char* what);
+// Compute units of the current device (asked of the runtime once per device; 256, an MI355X's,
+// if it will not say).  Launch plans count blocks against this, not against a constant.
+int kvc_device_compute_units(void);

@@ -29,6 +29,24 @@ int kvc_check_launch(const char* what) {
   return 0;
 }
 
+int kvc_device_compute_units(void) {
+  constexpr int kMaxDevices = 64;
+  static int cached[kMaxDevices];  // 0: not asked yet
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return 256;
+  if (cached[device] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) {
+      (void)hipGetLastError();
+      n = 256;
+    }
+    cached[device] = n;
+  }
+  return cached[device];
+}
+
+extern "C" int kvc_compute_units(void) { return kvc_device_compute_units(); }
+
 extern "C" const char* kvc_last_error(void) { return g_last_error.c_str(); }
 extern "C" int kvc_version(void) { return 1; }
 
@@ -37,7 +55,7 @@ static inline hipStream_t S(kvc_stream s) { return reinterpret_cast<hipStream_t>
 // ------------------------------------------------------------------------ embedding
 template <typename T>
 __global__ void embed_kernel(float* __restrict__ residual, const T* __restrict__ table,
-                             const int32_t* __restrict__ ids, int H, int V) {
+                             const int32_t* __restrict__ ids, int H, int V, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   float* out = residual + static_cast<int64_t>(t) * H;
@@ -46,17 +64,74 @@ __global__ void embed_kernel(float* __restrict__ residual, const T* __restrict__
     return;
   }
   const T* row = table + static_cast<int64_t>(id) * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_float(row[i]);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_float(row[i]) * scale;
 }
 
 extern "C" int kvc_embed(float* residual, const void* table, const int32_t* ids, int T, int H,
-                         int V, int dtype, kvc_stream stream) {
+                         int V, int dtype, float scale, kvc_stream stream) {
   if (T < 0 || H <= 0 || V <= 0) return kvc_fail("kvc_embed: bad sizes");
   if (T == 0) return 0;
   KVC_DISPATCH_DTYPE(dtype, Tp, hipLaunchKernelGGL(embed_kernel<Tp>, dim3(T), dim3(256), 0,
                                                    S(stream), residual,
-                                                   static_cast<const Tp*>(table), ids, H, V));
+                                                   static_cast<const Tp*>(table), ids, H, V, scale));
   return kvc_check_launch("kvc_embed");
+}
+
+// ------------------------------------------------------------- logits after the head
+// x = logits + bias; x = cap * tanh(x / cap) when cap > 0; x *= scale.
+template <typename TB>
+__global__ void logits_finish_kernel(float* __restrict__ logits, int V, int64_t row_stride,
+                                     const TB* __restrict__ bias, float soft_cap, float scale) {
+  float* row = logits + static_cast<int64_t>(blockIdx.y) * row_stride;
+  const int v = blockIdx.x * blockDim.x + threadIdx.x;
+  if (v >= V) return;
+  float x = row[v];
+  if (bias != nullptr) x += to_float(bias[v]);
+  if (soft_cap > 0.f) x = tanhf(x / soft_cap) * soft_cap;
+  row[v] = x * scale;
+}
+
+extern "C" int kvc_logits_finish(float* logits, int S_, int V, int64_t row_stride, const void* bias,
+                                 int bias_dtype, float soft_cap, float scale, kvc_stream stream) {
+  if (S_ < 0 || V <= 0 || row_stride < V || S_ > 65535)
+    return kvc_fail("kvc_logits_finish: bad sizes (at most 65535 rows)");
+  if (soft_cap < 0.f) return kvc_fail("kvc_logits_finish: the soft cap must not be negative");
+  if (S_ == 0) return 0;
+  const dim3 grid((V + 255) / 256, S_);
+  KVC_DISPATCH_DTYPE(bias_dtype, Tb,
+                     hipLaunchKernelGGL(logits_finish_kernel<Tb>, grid, dim3(256), 0, S(stream), logits,
+                                        V, row_stride, static_cast<const Tb*>(bias), soft_cap, scale));
+  return kvc_check_launch("kvc_logits_finish");
+}
+
+// ------------------------------------------------------------------- filling of pages
+// Every element of the listed pages, in all `outer` planes of a cache group's storage
+// [outer, num_pages, page_elems], becomes the 16- or 32-bit pattern `bits`.
+template <typename U>
+__global__ void fill_pages_kernel(U* __restrict__ base, const int32_t* __restrict__ pages,
+                                  int page_stride, int num_pages, int64_t page_elems, U bits) {
+  const int page = pages[static_cast<int64_t>(blockIdx.x) * page_stride];
+  if (page <= 0 || page >= num_pages) return;  // the null page is nobody's
+  U* dst = base + (static_cast<int64_t>(blockIdx.y) * num_pages + page) * page_elems;
+  for (int64_t i = threadIdx.x; i < page_elems; i += blockDim.x) dst[i] = bits;
+}
+
+extern "C" int kvc_fill_pages(void* storage, const int32_t* pages, int page_stride, int n, int outer,
+                              int num_pages, int64_t page_elems, int elem_bytes, uint32_t bits,
+                              kvc_stream stream) {
+  if (n < 0 || page_stride <= 0 || outer <= 0 || outer > 65535 || num_pages <= 0 || page_elems <= 0)
+    return kvc_fail("kvc_fill_pages: bad sizes");
+  if (elem_bytes != 2 && elem_bytes != 4) return kvc_fail("kvc_fill_pages: elements of 2 or 4 bytes");
+  if (n == 0) return 0;
+  const dim3 grid(n, outer);
+  if (elem_bytes == 2)
+    hipLaunchKernelGGL(fill_pages_kernel<uint16_t>, grid, dim3(256), 0, S(stream),
+                       static_cast<uint16_t*>(storage), pages, page_stride, num_pages, page_elems,
+                       static_cast<uint16_t>(bits));
+  else
+    hipLaunchKernelGGL(fill_pages_kernel<uint32_t>, grid, dim3(256), 0, S(stream),
+                       static_cast<uint32_t*>(storage), pages, page_stride, num_pages, page_elems, bits);
+  return kvc_check_launch("kvc_fill_pages");
 }
 
 // -------------------------------------------------------------------------- RMSNorm

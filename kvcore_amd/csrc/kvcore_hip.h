@@ -16,10 +16,33 @@ typedef void* kvc_stream;
 
 const char* kvc_last_error(void);
 int kvc_version(void);
+// Compute units of the current device: what the launch plans of the attention kernels count
+// blocks against.
+int kvc_compute_units(void);
 
-// residual[t, :] = float(table[ids[t], :]); an id outside [0, V) gives a NaN row.
+// residual[t, :] = float(table[ids[t], :]) * scale; an id outside [0, V) gives a NaN row.
 int kvc_embed(float* residual, const void* table, const int32_t* ids, int T, int H, int V,
-              int dtype, kvc_stream stream);
+              int dtype, float scale, kvc_stream stream);
+
+// What a head may do to its logits [S, V] (float32, rows row_stride apart) after the product,
+// in place: x += bias[v] (bias of bias_dtype, or null); x = soft_cap * tanh(x / soft_cap) when
+// soft_cap > 0; x *= scale.
+int kvc_logits_finish(float* logits, int S, int V, int64_t row_stride, const void* bias,
+                      int bias_dtype, float soft_cap, float scale, kvc_stream stream);
+
+// Every element of the pages pages[i * page_stride], i < n, in all `outer` planes of a cache
+// group's storage [outer, num_pages, page_elems] (elements of elem_bytes = 2 or 4) becomes the
+// bit pattern `bits` (its low 16 bits for 2-byte elements): zeros, or a NaN that makes a read
+// of a slot nobody wrote show in the logits.  The null page (0) and ids outside the pool are
+// skipped.  Reference: kvcore/model/model_runner.py:646-657 zeroes new blocks with index_fill_.
+int kvc_fill_pages(void* storage, const int32_t* pages, int page_stride, int n, int outer,
+                   int num_pages, int64_t page_elems, int elem_bytes, uint32_t bits, kvc_stream stream);
+
+// out[i] = mean + std * z_i for i < n, out of dtype: z_i is a standard normal variate that is a
+// function of (seed_lo, seed_hi, i) alone, worked out in single float32 operations that a host
+// program can repeat bit for bit (see random_fill.hip).
+int kvc_fill_normal(void* out, int64_t n, int dtype, uint32_t seed_lo, uint32_t seed_hi, float mean,
+                    float std, kvc_stream stream);
 
 // residual += delta (skipped when delta is null); out = weight * residual *
 // rsqrt(mean(residual^2) + eps), rounded to dt.  residual stays float32.
@@ -96,8 +119,12 @@ int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* 
 // kernel one dependent load.
 // kvc_decode_attention_supported tells whether a shape is served (else use
 // kvc_paged_attention); kvc_decode_attention_waves how many waves share a block's key range.
+// kvc_decode_attention_max_table: the widest block table (entries per request) whose page ids
+// for one split still fit in a block's LDS; a wider one is refused, so engines check it when
+// they are built.
 int kvc_decode_attention_supported(int nh, int nkv, int d, int page_size, int dtype);
 int kvc_decode_attention_waves(int nh, int nkv, int d);
+int kvc_decode_attention_max_table(int nh, int nkv, int d);
 int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* qkv,
                          int64_t qkv_stride, void* k_cache, void* v_cache, const int32_t* table,
                          int table_stride, const int32_t* positions, const int32_t* token_req,

@@ -13,9 +13,9 @@ from typing import Any, Mapping, Sequence
 
 import torch
 
-from kvcore_amd.cache.kv_manager import GroupConfig, KVManager, cdiv
+from kvcore_amd.cache.kv_manager import KVManager, cdiv, plan_groups
 from kvcore_amd.config.engine_config import KVCoreConfig, canonical_dtype
-from kvcore_amd.config.model_config import read_config_json
+from kvcore_amd.config.model_config import read_config_json, read_generation_eos
 from kvcore_amd.sampling.params import SamplingParams
 from kvcore_amd.sampling.sampler import PendingTokens, Sampler, SamplingRow
 
@@ -89,21 +89,32 @@ class EngineCore:
         cache = config.cache_config
         self.max_model_len = config.model_config.max_model_len or model.spec.max_position_embeddings
         self.page_size = cache.block_size
+        # ``num_pages`` counts pages of ``block_size`` tokens (with the null page); a cache
+        # group whose mixers want another page size holds the same number of tokens
         self.num_pages = self._decide_num_pages()
-        groups = [GroupConfig(self.page_size, self.num_pages, g.need.window) for g in model.cache_groups]
-        self.kv_manager = KVManager(groups, max_num_seqs=sched.max_num_seqs, max_model_len=self.max_model_len)
+        self.group_configs = plan_groups([g.need for g in model.cache_groups], self.page_size, self.num_pages)
+        self.kv_manager = KVManager(self.group_configs, max_num_seqs=sched.max_num_seqs,
+                                    max_model_len=self.max_model_len, track_freed=cache.poison_pages)
         self.scheduler = Scheduler(sched, self.kv_manager, max_model_len=self.max_model_len)
-        self.runner = ModelRunner(model, page_size=self.page_size, num_pages=self.num_pages,
+        self.runner = ModelRunner(model, page_size=[g.page_size for g in self.group_configs],
+                                  num_pages=[g.num_pages for g in self.group_configs],
                                   max_num_seqs=sched.max_num_seqs,
                                   max_num_tokens=sched.max_num_scheduled_tokens,
                                   max_model_len=self.max_model_len,
-                                  use_hip_graphs=config.device_config.use_hip_graphs)
+                                  use_hip_graphs=config.device_config.use_hip_graphs,
+                                  poison_pages=cache.poison_pages)
+        if cache.poison_pages:
+            self.runner.fill_cache(float("nan"))
         self.sampler = Sampler(device, sched.max_num_seqs, engine_seed=config.load_config.seed)
         self.tokenizer_manager = None
         if model_json:
             self.tokenizer_manager = TokenizerManager.from_model_source(
                 config.model_config.tokenizer or config.model_config.model)
+        # stop ids: config.json's, generation_config.json's and the tokenizer's, joined
+        # (reference: engine_core.py:209-217 joins the tokenizer's and the config's)
         self.stop_token_ids = set(model.spec.eos_token_ids)
+        if model_json:
+            self.stop_token_ids |= set(read_generation_eos(config.model_config.model))
         if self.tokenizer_manager is not None:
             self.stop_token_ids |= self.tokenizer_manager.get_stop_token_ids()
         self._seeds: dict[str, int] = {}
@@ -114,9 +125,10 @@ class EngineCore:
 
     # ---------------------------------------------------------------------- capacity
     def bytes_per_page(self) -> int:
-        esize = torch.empty((), dtype=self.dtype).element_size()
+        """Bytes that ``block_size`` tokens take in the cache, over all groups and planes."""
         return sum(g.num_planes * 2 * g.need.num_kv_heads * self.page_size * g.need.head_dim
-                   for g in self.model.cache_groups) * esize
+                   * torch.empty((), dtype=g.need.dtype or self.dtype).element_size()
+                   for g in self.model.cache_groups)
 
     def _decide_num_pages(self) -> int:
         """An explicit ``num_gpu_blocks`` wins.  Otherwise: free device memory times the
@@ -239,6 +251,8 @@ class EngineCore:
             if s.samples:
                 rows.append(SamplingRow(s.sampling_params, self._seeds[s.request_id], s.num_output_tokens))
                 row_ids.append(s.request_id)
+        if self.runner.poison_pages:
+            self.runner.poison(self.kv_manager.drain_freed())
         step_out = self.runner.step(entries, device_tokens)
         tokens = self.sampler.launch(step_out.logits, rows) if rows else PendingTokens(None, 0)
         return _Flight(out, row_ids, tokens)

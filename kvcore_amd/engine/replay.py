@@ -11,7 +11,7 @@ from typing import Any, Mapping
 
 import torch
 
-from kvcore_amd.cache.kv_manager import GroupConfig, KVManager
+from kvcore_amd.cache.kv_manager import KVManager, plan_groups
 
 from .runner import ModelRunner, StepEntry, StepOutput, build_model
 
@@ -25,13 +25,14 @@ class TraceSession:
         capacity = -(-max_tokens // 64) * 64
         self.capacity = capacity
         self.num_pages = -(-capacity // page) + 1  # + the null page
-        groups = [GroupConfig(page, self.num_pages, g.need.window) for g in self.model.cache_groups]
+        groups = plan_groups([g.need for g in self.model.cache_groups], page, self.num_pages)
         self.manager = KVManager(groups, max_num_seqs=max_num_seqs, max_model_len=capacity,
-                                 shuffle_seed=shuffle_pages)
-        self.runner = ModelRunner(self.model, page_size=page, num_pages=self.num_pages,
+                                 shuffle_seed=shuffle_pages, track_freed=poison_cache)
+        self.runner = ModelRunner(self.model, page_size=[g.page_size for g in groups],
+                                  num_pages=[g.num_pages for g in groups],
                                   max_num_seqs=max_num_seqs, max_num_tokens=capacity,
-                                  max_model_len=capacity)
-        if poison_cache:
+                                  max_model_len=capacity, poison_pages=poison_cache)
+        if poison_cache:  # the whole cache now, every page again when it is taken or given back
             self.runner.fill_cache(float("nan"))
         self.computed: dict[str, int] = {}
 
@@ -60,6 +61,8 @@ class TraceSession:
                                      self.manager.released_counts(rid)))
         out = None
         if entries:
+            if self.runner.poison_pages:
+                self.runner.poison(self.manager.drain_freed())
             out = self.runner.step(entries)
             for e in entries:
                 self.computed[e.request_id] += len(e.tokens)

@@ -56,6 +56,10 @@ class Request:
         self.num_computed_tokens = 0
         self.status = RequestStatus.WAITING
         self.num_preemptions = 0
+        # how many leading tokens count as "prompt" for the scheduler's limits on requests
+        # that are still prefilling: the prompt, or, after a preemption, the prompt and the
+        # output so far, which are computed again as one prompt
+        self.num_prefill_tokens = len(self.prompt_token_ids)
 
     @property
     def num_prompt_tokens(self) -> int:

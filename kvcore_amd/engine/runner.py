@@ -31,6 +31,7 @@ import torch
 from kvcore_amd.config.model_config import read_config_json
 from kvcore_amd.models.decoder import DecoderModel
 from kvcore_amd.ops import library as ops
+from kvcore_amd.parts.base import RunLimits
 from kvcore_amd.registry import resolve_architecture
 
 from .context import CacheGroupView, StepBuffers, StepContext
@@ -89,32 +90,47 @@ class ModelRunner:
     """Owns the device side of the cache (planes, block tables, state arrays), the step
     buffers and the model; runs steps."""
 
-    def __init__(self, model: DecoderModel, *, page_size: int, num_pages: int | Sequence[int],
-                 max_num_seqs: int, max_num_tokens: int, max_model_len: int,
-                 use_hip_graphs: bool = True) -> None:
+    def __init__(self, model: DecoderModel, *, page_size: int | Sequence[int],
+                 num_pages: int | Sequence[int], max_num_seqs: int, max_num_tokens: int,
+                 max_model_len: int, use_hip_graphs: bool = True, poison_pages: bool = False) -> None:
+        """``page_size`` and ``num_pages``: one value for every cache group, or one per group
+        (``num_pages`` counts the null page).  ``poison_pages``: a debugging aid that fills
+        every page with NaN when it is first listed for a request (see ``poison``)."""
         ops.load()  # fail here, loudly, if the kernels are not there
         if model.device.type != "cuda":
             raise RuntimeError("kvcore_amd runs on a GPU only; there is no CPU path")
         self.model = model
         self.device = model.device
         self.dtype = model.dtype
-        self.page_size = page_size
         self.max_num_seqs = max_num_seqs
         self.max_num_tokens = max_num_tokens
         self.max_model_len = max_model_len
-        self.max_pages_per_seq = -(-max_model_len // page_size)
         n_groups = len(model.cache_groups)
+        self.page_sizes = [page_size] * n_groups if isinstance(page_size, int) else list(page_size)
         self.num_pages = [num_pages] * n_groups if isinstance(num_pages, int) else list(num_pages)
-        if len(self.num_pages) != n_groups:
-            raise ValueError("num_pages must give one count per cache group")
+        if len(self.num_pages) != n_groups or len(self.page_sizes) != n_groups:
+            raise ValueError("page_size and num_pages must give one value per cache group")
+        self.poison_pages = poison_pages
 
         self.groups: list[CacheGroupView] = []
-        for gs, pages in zip(model.cache_groups, self.num_pages):
-            kv = torch.empty((gs.num_planes, 2, pages, gs.need.num_kv_heads, page_size,
-                              gs.need.head_dim), dtype=self.dtype, device=self.device)
-            table = torch.zeros((max_num_seqs, self.max_pages_per_seq), dtype=torch.int32,
+        for gs, size, pages in zip(model.cache_groups, self.page_sizes, self.num_pages):
+            if gs.need.page_size is not None and gs.need.page_size != size:
+                raise ValueError(f"a cache group wants pages of {gs.need.page_size} tokens, got {size}")
+            kv = torch.empty((gs.num_planes, 2, pages, gs.need.num_kv_heads, size, gs.need.head_dim),
+                             dtype=gs.need.dtype or self.dtype, device=self.device)
+            table = torch.zeros((max_num_seqs, -(-max_model_len // size)), dtype=torch.int32,
                                 device=self.device)
-            self.groups.append(CacheGroupView(kv, table, page_size, gs.need.window))
+            self.groups.append(CacheGroupView(kv, table, size, gs.need.window))
+        # every part learns the sizes it will run at and may refuse them now, with a message,
+        # rather than in the middle of a generation
+        for call in model.calls:
+            limits = RunLimits(max_num_seqs, max_num_tokens, max_model_len)
+            if call.group_index is not None:
+                size = self.page_sizes[call.group_index]
+                limits = RunLimits(max_num_seqs, max_num_tokens, max_model_len, size, -(-max_model_len // size))
+            block = model.blocks[call.layer_index]
+            for part in (block, *block.children().values()):
+                part.check_limits(limits)
         self.states = [
             torch.zeros((max_num_seqs, *sa.need.shape), dtype=sa.need.dtype, device=self.device)
             for sa in model.state_arrays
@@ -182,15 +198,26 @@ class ModelRunner:
         """A request left its slot.  The next owner's pages are synced from scratch."""
         self._slot_owner[slot] = None
 
+    def poison(self, pages: Sequence[Sequence[int]]) -> None:
+        """Fill the listed pages (one list per cache group) with NaN on the stream, behind the
+        steps launched so far: for pages that were given back, so that a table row that still
+        names them shows in the logits.  A debugging aid (the reference zeroes new blocks,
+        kvcore/model/model_runner.py:646-657; here nothing needs it for correctness, since
+        every kernel reads only the slots its request has written)."""
+        for grp, ids in zip(self.groups, pages):
+            ids = [p for p in ids if p > 0]
+            if ids:
+                dev = torch.tensor(ids, dtype=torch.int32, device=self.device)
+                ops.fill_pages(grp.kv, dev, len(ids), float("nan"))
+
     def fill_cache(self, value: float) -> None:
         """Overwrite every cache plane (tests fill with NaN so that a read outside a
         request's own slots shows in the logits)."""
         for g in self.groups:
             g.kv.fill_(value)
 
-    def cache_bytes_per_page(self) -> int:
-        return sum(gs.num_planes * 2 * gs.need.num_kv_heads * self.page_size * gs.need.head_dim
-                   for gs in self.model.cache_groups) * torch.empty((), dtype=self.dtype).element_size()
+    def cache_bytes(self) -> int:
+        return sum(g.kv.numel() * g.kv.element_size() for g in self.groups)
 
     def _table_updates(self, entries: Sequence[StepEntry]) -> list[list[int]]:
         """Per group, flat triples (slot, index, page) that bring the device tables up to
@@ -269,9 +296,8 @@ class ModelRunner:
                 raise ValueError(f"step exceeds max_num_tokens={self.max_num_tokens}")
             if min(slot_list) < 0 or max(slot_list) >= self.max_num_seqs or len(set(slot_list)) != R:
                 raise ValueError("a slot is invalid or used twice")
-            page = self.page_size
             for e in entries:
-                for g_pages in e.pages:
+                for g_pages, page in zip(e.pages, self.page_sizes):
                     if len(g_pages) * page <= e.start:
                         raise ValueError(f"request {e.request_id!r}: {len(g_pages)} pages do not hold "
                                          f"{e.start + 1} tokens")
@@ -307,7 +333,7 @@ class ModelRunner:
                 raise ValueError(f"request {e.request_id!r}: slot {e.slot} is invalid or used twice")
             seen_slots.add(e.slot)
             for g, grp in enumerate(self.groups):
-                if len(e.pages[g]) * self.page_size < end:
+                if len(e.pages[g]) * grp.page_size < end:
                     raise ValueError(f"request {e.request_id!r}: {len(e.pages[g])} pages do not hold "
                                      f"{end} tokens")
             toks = np.asarray(e.tokens, dtype=np.int64)
@@ -365,7 +391,10 @@ class ModelRunner:
             self._dev["token_ids"][:R].copy_(device_tokens[:R])
         for g, (off, count) in enumerate(upd_counts):
             if count:
-                ops.table_update(self.groups[g].table, self._meta_dev[off:off + 3 * count], count)
+                triples = self._meta_dev[off:off + 3 * count]
+                ops.table_update(self.groups[g].table, triples, count)
+                if self.poison_pages:  # the pages listed for the first time: third of each triple
+                    ops.fill_pages(self.groups[g].kv, triples[2:], count, float("nan"), stride=3)
 
         ids = [e.request_id for e in entries]
         if bucket:

@@ -151,11 +151,13 @@ class Scheduler:
 
     # ------------------------------------------------------------------------ helpers
     def _is_prefill(self, request: Request) -> bool:
-        return request.num_computed_tokens < request.num_prompt_tokens
+        """Still in its prompt (scheduler.py:541-543), where "prompt" includes, after a
+        preemption, the output that is computed again with it."""
+        return request.num_computed_tokens < request.num_prefill_tokens
 
     def _is_long_prefill(self, request: Request) -> bool:
         threshold = self.config.long_prefill_token_threshold
-        return threshold > 0 and request.num_prompt_tokens >= threshold
+        return threshold > 0 and request.num_prefill_tokens >= threshold
 
     def _can_schedule_partial_prefill(self, request: Request, num_partial: int, num_long: int) -> bool:
         if num_partial >= self.config.max_num_partial_prefills:
@@ -173,6 +175,7 @@ class Scheduler:
         self.kv_manager.free(request.request_id)
         request.status = RequestStatus.PREEMPTED
         request.num_computed_tokens = 0
+        request.num_prefill_tokens = request.num_tokens  # all of it is a prompt now
         request.num_preemptions += 1
         self.num_preemptions += 1
         self.running.remove(request)

@@ -15,7 +15,6 @@ from kvcore_amd.engine.context import LayerCall, StepContext
 from kvcore_amd.ops import library as ops
 from kvcore_amd.parts import base as parts
 from kvcore_amd.parts.base import CacheNeed, ParamSpec, Part, Runtime, StateNeed
-from kvcore_amd.parts.embedding import OutputHead, TokenEmbedding
 
 from .spec import ModelSpec
 
@@ -42,6 +41,43 @@ class BoundParam:
     tensor: torch.Tensor
 
 
+@dataclass
+class BuiltParts:
+    positions: list
+    embed: parts.Embedding
+    head: parts.Head
+    final_norm: parts.Norm
+    blocks: list
+    owned: list  # (checkpoint prefix, part), in the order parameters are declared
+
+
+def build_parts(spec: ModelSpec) -> BuiltParts:
+    """Every part that ``spec`` names, from the registries, with its checkpoint prefix.
+    Nothing is allocated: the loader uses this to learn a model's checkpoint layout."""
+    positions = [parts.POSITION_ENCODINGS.build(p) for p in spec.positions]
+    embed = parts.EMBEDDINGS.build(spec.resolved_embedding())
+    head = parts.HEADS.build(spec.resolved_head())
+    final_norm = parts.NORMS.build(spec.final_norm)
+    blocks: list[parts.Block] = []
+    for layer in spec.layers:
+        position = None if layer.position is None else positions[layer.position]
+        mixer = parts.MIXERS.build(layer.mixer, position=position)
+        ffn = parts.FEED_FORWARDS.build(layer.ffn)
+        norms = {name: parts.NORMS.build(ns) for name, ns in layer.norms.items()}
+        blocks.append(parts.BLOCKS.build(layer.block, mixer=mixer, ffn=ffn, norms=norms))
+    owned: list[tuple[str, Part]] = [(spec.embed_prefix, embed), (spec.final_norm_prefix, final_norm),
+                                     (spec.head_prefix, head)]
+    if spec.position_prefixes and len(spec.position_prefixes) != len(positions):
+        raise ValueError("position_prefixes must name every position encoding")
+    for i, pe in enumerate(positions):
+        prefix = spec.position_prefixes[i] if spec.position_prefixes else f"model.positions.{i}"
+        owned.append((prefix, pe))
+    for layer, block in zip(spec.layers, blocks):
+        for sub, part in block.children().items():
+            owned.append((f"{layer.prefix}.{sub}", part))
+    return BuiltParts(positions, embed, head, final_norm, blocks, owned)
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, dtype: torch.dtype, device: torch.device | str) -> None:
         self.spec = spec
@@ -49,30 +85,13 @@ class DecoderModel:
         self.dtype = dtype
         self.device = self.runtime.device
 
-        self.positions = [parts.POSITION_ENCODINGS.build(p) for p in spec.positions]
-        self.embed = TokenEmbedding(vocab_size=spec.vocab_size, hidden_size=spec.hidden_size)
-        self.head = OutputHead(vocab_size=spec.vocab_size, hidden_size=spec.hidden_size,
-                               tied=spec.tie_word_embeddings)
-        self.final_norm = parts.NORMS.build(spec.final_norm)
-        self.blocks: list[parts.Block] = []
-        for layer in spec.layers:
-            position = None if layer.position is None else self.positions[layer.position]
-            mixer = parts.MIXERS.build(layer.mixer, position=position)
-            ffn = parts.FEED_FORWARDS.build(layer.ffn)
-            norms = {name: parts.NORMS.build(ns) for name, ns in layer.norms.items()}
-            self.blocks.append(parts.BLOCKS.build(layer.block, mixer=mixer, ffn=ffn, norms=norms))
-
-        self._owned: list[tuple[str, Part]] = [(spec.embed_prefix, self.embed),
-                                               (spec.final_norm_prefix, self.final_norm),
-                                               (spec.head_prefix, self.head)]
-        if spec.position_prefixes and len(spec.position_prefixes) != len(self.positions):
-            raise ValueError("position_prefixes must name every position encoding")
-        for i, pe in enumerate(self.positions):
-            prefix = spec.position_prefixes[i] if spec.position_prefixes else f"model.positions.{i}"
-            self._owned.append((prefix, pe))
-        for layer, block in zip(spec.layers, self.blocks):
-            for sub, part in block.children().items():
-                self._owned.append((f"{layer.prefix}.{sub}", part))
+        built = build_parts(spec)
+        self.positions = built.positions
+        self.embed = built.embed
+        self.head = built.head
+        self.final_norm = built.final_norm
+        self.blocks = built.blocks
+        self._owned = built.owned
         for _, part in self._owned:
             part.setup(self.runtime)
 
@@ -135,8 +154,10 @@ class DecoderModel:
                 self.params[full] = BoundParam(full, prefix, ps, t)
                 local[ps.name] = t
             part.bind(local)
-        if self.spec.tie_word_embeddings:
-            self.head.bind({"weight": self.embed.params["weight"]})
+        if self.head.tied:
+            if "weight" not in self.embed.params:
+                raise ValueError("a tied head needs an embedding with a parameter named 'weight'")
+            self.head.bind({**self.head.params, "weight": self.embed.params["weight"]})
 
     def checkpoint_map(self) -> dict[str, tuple[BoundParam, int, int]]:
         """Checkpoint tensor name -> (parameter, first row, rows)."""
@@ -149,7 +170,7 @@ class DecoderModel:
     def optional_checkpoint_names(self) -> set[str]:
         """Names a file may hold that are not read: a tied head's own matrix
         (reference: kvcore/model/model_utils.py:51-53)."""
-        if self.spec.tie_word_embeddings:
+        if self.head.tied:
             return {f"{self.spec.head_prefix}.weight"}
         return set()
 

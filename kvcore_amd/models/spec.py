@@ -41,6 +41,11 @@ class ModelSpec:
     positions: tuple[PartSpec, ...] = ()
     schedule: tuple[ScheduleEntry, ...] = ()
     tie_word_embeddings: bool = False
+    # the embedding and the head, chosen by kind like every other part; None stands for the
+    # plain token embedding and the linear head (tied as ``tie_word_embeddings`` says) of
+    # this vocabulary and width
+    embedding: PartSpec | None = None
+    head: PartSpec | None = None
     eos_token_ids: tuple[int, ...] = ()
     # checkpoint prefixes of the position encodings' own parameters, one per entry of
     # ``positions`` (empty: "model.positions.<i>"; a rotary encoding has no parameters)
@@ -55,3 +60,12 @@ class ModelSpec:
 
     def resolved_schedule(self) -> tuple[ScheduleEntry, ...]:
         return self.schedule or tuple(ScheduleEntry(i) for i in range(len(self.layers)))
+
+    def resolved_embedding(self) -> PartSpec:
+        return self.embedding or PartSpec("token_embedding", {
+            "vocab_size": self.vocab_size, "hidden_size": self.hidden_size})
+
+    def resolved_head(self) -> PartSpec:
+        return self.head or PartSpec("linear_head", {
+            "vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
+            "tied": self.tie_word_embeddings})

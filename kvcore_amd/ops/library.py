@@ -32,7 +32,10 @@ class KernelError(RuntimeError):
 def _declare(lib: ctypes.CDLL) -> None:
     P, I, L, F = c_void_p, c_int, c_int64, c_float
     sigs = {
-        "kvc_embed": [P, P, P, I, I, I, I, P],
+        "kvc_embed": [P, P, P, I, I, I, I, F, P],
+        "kvc_logits_finish": [P, I, I, L, P, I, F, F, P],
+        "kvc_fill_pages": [P, P, I, I, I, I, L, I, ctypes.c_uint32, P],
+        "kvc_fill_normal": [P, L, I, ctypes.c_uint32, ctypes.c_uint32, F, F, P],
         "kvc_add_rmsnorm": [P, P, P, P, F, I, I, I, P],
         "kvc_add_slices_rmsnorm": [P, P, P, I, P, P, F, I, I, I, P],
         "kvc_rmsnorm": [P, P, P, F, I, I, L, L, I, P],
@@ -47,6 +50,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
                                  F, I, I, P],
         "kvc_decode_attention_waves": [I, I, I],
+        "kvc_decode_attention_max_table": [I, I, I],
         "kvc_decode_attention_supported": [I, I, I, I, I],
         "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, P, I,
                                   P, P, I, I, P],
@@ -72,6 +76,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.kvc_last_error.restype = ctypes.c_char_p
     lib.kvc_last_error.argtypes = []
     lib.kvc_version.restype = c_int
+    lib.kvc_compute_units.restype = c_int
+    lib.kvc_compute_units.argtypes = []
     lib.kvc_argmax_static_capacity.restype = c_int
     lib.kvc_argmax_static_capacity.argtypes = []
 
@@ -134,14 +140,59 @@ def _code(t: torch.Tensor, name: str) -> int:
 
 
 # ------------------------------------------------------------------------ wrappers
-def embed(residual: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+def embed(residual: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> None:
+    """``residual[t] = float(table[ids[t]]) * scale``; an id outside the table gives a NaN row."""
     T, H = residual.shape
     V = table.shape[0]
     if table.shape[1] != H or ids.numel() != T:
         raise KernelError("embed: shapes do not match")
     _check(load().kvc_embed(_dev(residual, "residual", torch.float32), _dev(table, "table"),
-                            _dev(ids, "ids", torch.int32), T, H, V, _code(table, "table"), _stream()),
-           "kvc_embed")
+                            _dev(ids, "ids", torch.int32), T, H, V, _code(table, "table"), float(scale),
+                            _stream()), "kvc_embed")
+
+
+def logits_finish(logits: torch.Tensor, bias: torch.Tensor | None = None, soft_cap: float = 0.0,
+                  scale: float = 1.0) -> None:
+    """In place on float32 ``logits [S, V]``: ``+ bias``, then ``soft_cap * tanh(x / soft_cap)``
+    when ``soft_cap > 0``, then ``* scale`` (the order of kvcore/sample/logits_processor.py:50-54)."""
+    S, V = logits.shape
+    if logits.dtype != torch.float32 or not logits.is_cuda or logits.stride(1) != 1:
+        raise KernelError("logits_finish: expects float32 GPU logits [S, V]")
+    if bias is not None and bias.shape != (V,):
+        raise KernelError("logits_finish: bias must be [V]")
+    _check(load().kvc_logits_finish(logits.data_ptr(), S, V, logits.stride(0),
+                                    None if bias is None else _dev(bias, "bias"),
+                                    0 if bias is None else _code(bias, "bias"), float(soft_cap),
+                                    float(scale), _stream()), "kvc_logits_finish")
+
+
+def fill_pages(storage: torch.Tensor, pages: torch.Tensor, n: int, value: float, stride: int = 1) -> None:
+    """``storage`` is a cache group's ``[..., num_pages, kv_heads, page_size, head_dim]``
+    (contiguous, float32 or bfloat16); every element of the pages ``pages[i * stride]``,
+    ``i < n`` (int32 on the device), in all leading planes becomes ``value`` (0 or NaN as a
+    rule); the null page is skipped."""
+    if storage.dim() < 4 or not storage.is_contiguous():
+        raise KernelError("fill_pages: storage must be contiguous [..., pages, heads, page_size, d]")
+    if n > 0 and pages.numel() < (n - 1) * stride + 1:
+        raise KernelError("fill_pages: page list too short")
+    num_pages = storage.shape[-4]
+    page_elems = storage.shape[-3] * storage.shape[-2] * storage.shape[-1]
+    outer = storage.numel() // (num_pages * page_elems)
+    esize = storage.element_size()
+    probe = torch.tensor([value], dtype=storage.dtype)
+    bits = int(probe.view(torch.int16 if esize == 2 else torch.int32)[0]) & (0xFFFF if esize == 2 else 0xFFFFFFFF)
+    if pages.dtype != torch.int32 or not pages.is_cuda:
+        raise KernelError("fill_pages: pages must be int32 on the GPU")
+    _check(load().kvc_fill_pages(_dev(storage, "storage"), pages.data_ptr(), stride, n, outer,
+                                 num_pages, page_elems, esize, bits, _stream()), "kvc_fill_pages")
+
+
+def fill_normal(out: torch.Tensor, seed_lo: int, seed_hi: int, mean: float, std: float) -> None:
+    """``out`` (contiguous float32 or bfloat16 on the GPU) gets ``mean + std * z_i``, ``z_i`` the
+    normal variate of (seed_lo, seed_hi, i): the same bits as ``weights/random_normal.py``."""
+    _check(load().kvc_fill_normal(_dev(out, "out"), out.numel(), _code(out, "out"),
+                                  seed_lo & 0xFFFFFFFF, seed_hi & 0xFFFFFFFF, float(mean), float(std),
+                                  _stream()), "kvc_fill_normal")
 
 
 def add_rmsnorm(out: torch.Tensor, residual: torch.Tensor, delta: torch.Tensor | None,
@@ -277,6 +328,23 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
 
 def decode_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype: torch.dtype) -> bool:
     return bool(load().kvc_decode_attention_supported(nh, nkv, d, page_size, DTYPE_CODE.get(dtype, -1)))
+
+
+_COMPUTE_UNITS: int | None = None
+
+
+def compute_units() -> int:
+    """Compute units of the current GPU, which launch plans count their blocks against (256, an
+    MI355X's, where no GPU is visible: plans are also worked out on a host without one)."""
+    global _COMPUTE_UNITS
+    if _COMPUTE_UNITS is None:
+        _COMPUTE_UNITS = int(load().kvc_compute_units()) if torch.cuda.is_available() else 256
+    return _COMPUTE_UNITS
+
+
+def decode_attention_max_table(nh: int, nkv: int, d: int) -> int:
+    """The widest block table (entries per request) that :func:`decode_attention` serves."""
+    return int(load().kvc_decode_attention_max_table(nh, nkv, d))
 
 
 def decode_attention_waves(nh: int, nkv: int, d: int) -> int:
@@ -590,9 +658,13 @@ def _fused_skinny(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows
     return result
 
 
-def _skinny_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+def skinny_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the weight-streaming product for few rows takes these operands."""
     return (x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+_skinny_operands_ok = skinny_operands_ok
 
 
 def mid_slices_bound(N: int) -> int:
@@ -725,9 +797,9 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
 def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: torch.Tensor,
            bias: torch.Tensor | None = None) -> ScaledRows | None:
     """``out = x @ w.T (+ bias)``.  float32 runs the library's own true-float32 kernel.
-    bfloat16 with at most 64 rows runs the weight-streaming matrix-core kernel (float32
-    ``out`` allowed); more rows run the vendor matrix product through torch.  All sum in
-    float32.  With a :class:`ScaledRows` for ``x`` or a :class:`ResidualSink` for ``out``
+    bfloat16 with few rows runs the weight-streaming matrix-core kernel; more rows run the
+    vendor matrix product through torch.  All sum in float32, and a float32 ``out`` receives
+    the sums unrounded on either path.  With a :class:`ScaledRows` for ``x`` or a :class:`ResidualSink` for ``out``
     (few rows of bfloat16 only) the norm before or after the product is folded into it; a
     sink returns the :class:`ScaledRows` it made, or, in a step of 9 to 64 rows, where it
     finishes the norm itself, :class:`NormedRows`."""
@@ -749,15 +821,21 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
     skinny_ok = _skinny_operands_ok(x, w)
     # measured on MI355X (N x K of 4096..128256 x 4096..14336): the weight-streaming kernel
     # wins up to 8 rows everywhere, up to 16 rows unless K or N is very large and up to 32 rows
-    # for small matrices; it is also the only one that stores float32
-    if skinny_ok and (out.dtype == torch.float32 or M <= 8
-                      or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)
+    # for small matrices
+    if skinny_ok and (M <= 8 or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)
                       or (M <= 32 and K <= 4096 and N <= 4096)):
         gemm_skinny_bf16(out, x, w, bias)
         return
+    if out.dtype == torch.float32:
+        # the vendor product with float32 sums stored as they are (no rounding to bfloat16)
+        if out.stride(1) != 1 or not out.is_contiguous():
+            raise KernelError("linear: a float32 result of bfloat16 operands must be contiguous")
+        torch.mm(x, w.t(), out_dtype=torch.float32, out=out)
+        if bias is not None:
+            out.add_(bias.to(torch.float32))
+        return
     if out.dtype != torch.bfloat16:
-        raise KernelError("linear: float32 output of bfloat16 operands needs at most 64 rows, "
-                          "K a multiple of 8 and aligned operands")
+        raise KernelError(f"linear: unsupported result type {out.dtype}")
     if bias is None:
         torch.mm(x, w.t(), out=out)
     else:

@@ -15,18 +15,30 @@ from kvcore_amd.ops import library as ops
 from .base import CacheNeed, Mixer, ParamSource, ParamSpec, PositionEncoding, register_mixer
 
 
-DECODE_TARGET_BLOCKS = 256  # one block for each compute unit
 DECODE_MAX_SPLITS = 32
+
+
+def decode_target_blocks() -> int:
+    """Blocks a launch of the decode kernel wants: one for each compute unit."""
+    return ops.compute_units()
+
+
+def prefill_target_blocks() -> int:
+    """Blocks a launch of the kernel for portions wants: a compute unit holds two."""
+    return 2 * ops.compute_units()
 
 
 def prefill_split_rows(nkv: int, g: int) -> int:
     """An upper bound on tokens x splits when ``prefill_splits`` gives more than one split."""
     rows_tokens = max(128 // g, 1)
-    return 4 * PREFILL_TARGET_BLOCKS * rows_tokens // nkv + 2 * rows_tokens
+    return 4 * prefill_target_blocks() * rows_tokens // nkv + 2 * rows_tokens
 
 
-PREFILL_TARGET_BLOCKS = 512
-PREFILL_FEW_TILES = 128     # up to so many small tiles, splits go with small tiles
+def prefill_few_tiles() -> int:
+    """Up to so many small tiles (half the compute units), splits go with small tiles."""
+    return ops.compute_units() // 2
+
+
 PREFILL_MIN_KEYS = 256      # for steps of few tokens, whose partial results are small
 PREFILL_MIN_KEYS_MOST = 1024
 PREFILL_MAX_SPLITS = 32
@@ -48,19 +60,20 @@ def prefill_splits(T: int, nkv: int, g: int, max_query_len: int, max_seq_len: in
     keys = max_seq_len - min(T, max_query_len) // 2
     if window > 0:
         keys = min(keys, window + 2 * small_tokens)
-    if small_tiles <= PREFILL_FEW_TILES:
-        return max(1, min(-(-PREFILL_TARGET_BLOCKS // small_tiles), keys // PREFILL_MIN_KEYS, PREFILL_MAX_SPLITS))
-    if small_tiles <= PREFILL_TARGET_BLOCKS:
-        if small_tiles == PREFILL_TARGET_BLOCKS:
+    target = prefill_target_blocks()
+    if small_tiles <= prefill_few_tiles():
+        return max(1, min(-(-target // small_tiles), keys // PREFILL_MIN_KEYS, PREFILL_MAX_SPLITS))
+    if small_tiles <= target:
+        if small_tiles == target:
             return 1  # one small tile a block fills the chip as it is
         min_keys = min(max(T, PREFILL_MIN_KEYS), PREFILL_MIN_KEYS_MOST)
     else:
         min_keys = min(max(T // 2, PREFILL_MIN_KEYS), PREFILL_MIN_KEYS_MOST)
     rows_tokens = max(128 // g, 1)
     blocks = ((-(-T // rows_tokens)) + num_reqs) // 2 * nkv
-    if blocks >= PREFILL_TARGET_BLOCKS:
+    if blocks >= target:
         return 1
-    return max(1, min(-(-PREFILL_TARGET_BLOCKS // blocks), keys // min_keys, PREFILL_MAX_SPLITS))
+    return max(1, min(-(-target // blocks), keys // min_keys, PREFILL_MAX_SPLITS))
 
 
 def decode_splits(num_tokens: int, num_kv_heads: int, max_seq_len: int, waves: int,
@@ -71,14 +84,15 @@ def decode_splits(num_tokens: int, num_kv_heads: int, max_seq_len: int, waves: i
     enough to occupy every unit, as long as each wave still has a block of 16 keys."""
     keys = max_seq_len if window <= 0 else min(max_seq_len, window + 16)
     blocks = -(-keys // 16)
-    by_room = -(-DECODE_TARGET_BLOCKS // max(num_tokens * num_kv_heads, 1))
+    by_room = -(-decode_target_blocks() // max(num_tokens * num_kv_heads, 1))
     by_length = max(1, blocks // waves)
     return max(1, min(by_room, by_length, DECODE_MAX_SPLITS))
 
 
 class PagedAttention(Mixer):
     """``scale`` is a parameter (the reference fixes ``head_dim ** -0.5`` at
-    llama3.py:60); ``window`` 0 attends to every earlier token."""
+    llama3.py:60); ``window`` 0 attends to every earlier token; ``page_size`` asks for cache
+    pages of that many tokens for this layer's group (None: the engine's block size)."""
 
     @property
     def takes_scaled_rows(self) -> bool:  # x only goes into the qkv product
@@ -89,7 +103,7 @@ class PagedAttention(Mixer):
         return self.q_size % 8 == 0
 
     def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
-                 scale: float, bias: bool = False, window: int = 0,
+                 scale: float, bias: bool = False, window: int = 0, page_size: int | None = None,
                  position: PositionEncoding | None = None) -> None:
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
@@ -102,6 +116,7 @@ class PagedAttention(Mixer):
         self.scale = scale
         self.bias = bias
         self.window = window
+        self.page_size = page_size  # None: the engine's block size
         self.position = position
         self.q_size = num_heads * head_dim
         self.kv_size = num_kv_heads * head_dim
@@ -126,7 +141,21 @@ class PagedAttention(Mixer):
         return specs
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
+        return CacheNeed(self.num_kv_heads, self.head_dim, self.window, self.page_size)
+
+    def check_limits(self, limits) -> None:
+        """The decode kernel keeps the page ids of a split's key range in LDS; a block table
+        too wide for that is refused here, when the engine is built, not in a decode step."""
+        if self.runtime.dtype != torch.bfloat16 or not ops.decode_attention_supported(
+                self.num_heads, self.num_kv_heads, self.head_dim, limits.page_size, self.runtime.dtype):
+            return
+        widest = ops.decode_attention_max_table(self.num_heads, self.num_kv_heads, self.head_dim)
+        if limits.max_pages_per_seq > widest:
+            raise ValueError(
+                f"max_model_len={limits.max_model_len} with cache pages of {limits.page_size} tokens gives a "
+                f"block table of {limits.max_pages_per_seq} entries per request; the decode attention kernel "
+                f"serves at most {widest} for {self.num_heads} heads of {self.head_dim} over "
+                f"{self.num_kv_heads} kv heads: use a larger block_size or a smaller max_model_len")
 
     def product_weights(self) -> tuple[str, ...]:
         return ("qkv_proj.weight", "o_proj.weight")
@@ -159,7 +188,7 @@ class PagedAttention(Mixer):
             if nsplit > 1:
                 # tokens x splits is at most the blocks wanted per kv head plus the tokens: room
                 # for the largest at once, since a buffer that grows drops the graphs
-                most = (DECODE_TARGET_BLOCKS // self.num_kv_heads + 1 + max(T, ctx.buffers.seq_capacity)) \
+                most = (decode_target_blocks() // self.num_kv_heads + 1 + max(T, ctx.buffers.seq_capacity)) \
                     * self.num_heads
                 part_o = ctx.buffers.get("attn_part_o", T * self.num_heads * nsplit, self.head_dim,
                                          torch.float32, reserve=most)

@@ -60,11 +60,17 @@ class ParamSpec:
 class CacheNeed:
     """Paged memory that grows with the sequence: keys and values of ``num_kv_heads``
     heads of ``head_dim``.  ``window`` 0 keeps every token, ``w > 0`` only the last
-    ``w`` (pages wholly behind the window are given back during the request)."""
+    ``w`` (pages wholly behind the window are given back during the request).
+    ``page_size``: tokens per page if the mixer's kernels want a size of their own (None: the
+    engine's ``block_size``); ``dtype``: the cache's element type (None: the model's).  Mixers
+    with equal needs share a cache group; a group has its own page size, page count, pool,
+    storage and block table."""
 
     num_kv_heads: int
     head_dim: int
     window: int = 0
+    page_size: int | None = None
+    dtype: torch.dtype | None = None
 
 
 @dataclass(frozen=True)
@@ -73,6 +79,18 @@ class StateNeed:
 
     shape: tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+
+@dataclass(frozen=True)
+class RunLimits:
+    """The sizes a runner runs a part at.  ``page_size`` and ``max_pages_per_seq`` are those
+    of the part's cache group (0 if it has none)."""
+
+    max_num_seqs: int
+    max_num_tokens: int
+    max_model_len: int
+    page_size: int = 0
+    max_pages_per_seq: int = 0
 
 
 @dataclass(frozen=True)
@@ -105,6 +123,11 @@ class Part:
     def setup(self, runtime: Runtime) -> None:
         """Called once after construction, before parameters are bound."""
         self.runtime = runtime
+
+    def check_limits(self, limits: "RunLimits") -> None:
+        """Called when a runner is built around the model, with the sizes it will run at:
+        raise here, with a message that names the option to change, if a kernel of this part
+        cannot serve them (so that nothing is refused in the middle of a generation)."""
 
     def bind(self, params: dict[str, torch.Tensor]) -> None:
         """``params`` maps the local names of ``param_specs`` to device tensors."""
@@ -149,6 +172,26 @@ class RotaryTables:
     sin: torch.Tensor
     rot_dim: int
     interleaved: bool
+
+
+class Embedding(Part):
+    """Token ids to rows of the residual stream: ``forward`` writes ``residual [T, H]``
+    (float32) for ``token_ids [T]`` (int32 on the device).  A parameter named ``weight`` of
+    shape ``[vocab, hidden]`` is what a tied head shares."""
+
+    def forward(self, residual: torch.Tensor, token_ids: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """Normalised hidden rows to logits: ``forward`` writes float32 ``logits [S, V]`` from
+    ``hidden_rows [S, H]`` in the model dtype.  ``tied``: the head owns no matrix; the model
+    binds the embedding's ``weight`` to it under the same name."""
+
+    tied = False
+
+    def forward(self, logits: torch.Tensor, hidden_rows: torch.Tensor, ctx: "StepContext") -> None:
+        raise NotImplementedError
 
 
 class Mixer(Part):
@@ -253,6 +296,8 @@ FEED_FORWARDS = _Registry("feed-forward")
 NORMS = _Registry("norm")
 POSITION_ENCODINGS = _Registry("position encoding")
 BLOCKS = _Registry("block")
+EMBEDDINGS = _Registry("embedding")
+HEADS = _Registry("head")
 
 
 def register_mixer(kind: str, factory: Callable[..., Mixer], **kw: Any) -> None:
@@ -273,3 +318,11 @@ def register_position_encoding(kind: str, factory: Callable[..., PositionEncodin
 
 def register_block(kind: str, factory: Callable[..., Block], **kw: Any) -> None:
     BLOCKS.register(kind, factory, **kw)
+
+
+def register_embedding(kind: str, factory: Callable[..., Embedding], **kw: Any) -> None:
+    EMBEDDINGS.register(kind, factory, **kw)
+
+
+def register_head(kind: str, factory: Callable[..., Head], **kw: Any) -> None:
+    HEADS.register(kind, factory, **kw)

@@ -2,8 +2,9 @@
 
 Reference: kvcore/model/models/llama3.py:161-165,178-180 (a plain gather; the padding
 index has no effect on the forward pass) and :219-225,245-247 with
-kvcore/sample/logits_processor.py:30-54 (no bias; with tied embeddings the head's
-matrix is the embedding's).  Logits leave the head as float32.
+kvcore/sample/logits_processor.py:30-54 (the product, an optional bias, an optional soft
+cap ``cap * tanh(x / cap)``, then a scale; with tied embeddings the head's matrix is the
+embedding's).  Logits leave the head as float32 sums, whatever the number of rows.
 """
 
 from __future__ import annotations
@@ -12,54 +13,79 @@ import torch
 
 from kvcore_amd.ops import library as ops
 
-from .base import ParamSpec, Part
+from .base import Embedding, Head, ParamSpec, register_embedding, register_head
 
 
-class TokenEmbedding(Part):
-    def __init__(self, *, vocab_size: int, hidden_size: int) -> None:
+class TokenEmbedding(Embedding):
+    """``scale`` multiplies the embedded rows (1.0 for Llama; some architectures use
+    ``sqrt(hidden_size)``)."""
+
+    def __init__(self, *, vocab_size: int, hidden_size: int, scale: float = 1.0) -> None:
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
+        self.scale = float(scale)
 
     def param_specs(self) -> list[ParamSpec]:
         return [ParamSpec("weight", (self.vocab_size, self.hidden_size))]
 
     def forward(self, residual: torch.Tensor, token_ids: torch.Tensor) -> None:
-        ops.embed(residual, self.params["weight"], token_ids)
+        ops.embed(residual, self.params["weight"], token_ids, self.scale)
 
 
-class OutputHead(Part):
-    """``tied`` heads own no parameter; the model binds the embedding matrix to them."""
+class LinearHead(Head):
+    """``logits = hidden @ W.T (+ bias)``, then ``soft_cap * tanh(logits / soft_cap)`` if
+    ``soft_cap > 0``, then ``* logit_scale``.  ``tied`` heads own no matrix; the model binds
+    the embedding matrix to them."""
 
-    def __init__(self, *, vocab_size: int, hidden_size: int, tied: bool) -> None:
+    def __init__(self, *, vocab_size: int, hidden_size: int, tied: bool = False, bias: bool = False,
+                 logit_scale: float = 1.0, soft_cap: float = 0.0) -> None:
+        if soft_cap < 0:
+            raise ValueError(f"soft_cap must be positive when set, got {soft_cap}")
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.tied = tied
+        self.bias = bias
+        self.logit_scale = float(logit_scale)
+        self.soft_cap = float(soft_cap)
 
     def param_specs(self) -> list[ParamSpec]:
-        return [] if self.tied else [ParamSpec("weight", (self.vocab_size, self.hidden_size))]
+        specs = [] if self.tied else [ParamSpec("weight", (self.vocab_size, self.hidden_size))]
+        if self.bias:
+            specs.append(ParamSpec("bias", (self.vocab_size,), init="zeros"))
+        return specs
 
     def product_weights(self) -> tuple[str, ...]:
         return ("weight",)
 
     def forward(self, logits: torch.Tensor, hidden_rows: torch.Tensor, ctx) -> None:
         """``logits [S, V]`` float32 from ``hidden_rows [S, H]`` in the model dtype."""
+        self._product(logits, hidden_rows)
+        bias = self.params.get("bias")
+        if bias is not None or self.soft_cap > 0 or self.logit_scale != 1.0:
+            ops.logits_finish(logits, bias, self.soft_cap, self.logit_scale)
+
+    def _product(self, logits: torch.Tensor, hidden_rows: torch.Tensor) -> None:
         w = self.params["weight"]
         if hidden_rows.dtype == torch.float32:
             ops.linear(logits, hidden_rows, w)
             return
         S = hidden_rows.shape[0]
-        # measured at 128256 x 4096: the few-row kernel wins up to 12 rows, the kernel that
-        # shares the rows through LDS from 24 on (215 against 231 us at 64 rows), the vendor
-        # product with a conversion afterwards in between and beyond 64
-        if self.hidden_size % 8 == 0 and (S <= 12 or (S <= ops.SKINNY_PREFERRED_ROWS
-                                                       and self.vocab_size < 65536)):
-            ops.linear(logits, hidden_rows, w)  # float32 sums are stored without rounding
+        # Every branch stores the float32 sums unrounded, so a request's logits do not change
+        # their rounding with the number of rows beside it.  Measured at 128256 x 4096: the
+        # few-row kernel wins up to 12 rows, the kernel that shares the rows through LDS from
+        # 17 to 64 (215 against 231 us at 64 rows), the vendor product in between and beyond.
+        if ops.skinny_operands_ok(hidden_rows, w) and (
+                S <= 12 or (S <= ops.SKINNY_PREFERRED_ROWS and self.vocab_size < 65536)):
+            ops.gemm_skinny_bf16(logits, hidden_rows, w)
             return
         if ops.SKINNY_PREFERRED_ROWS < S <= ops.MID_ROWS and ops.mid_operands_ok(hidden_rows, w) \
                 and logits.stride(1) == 1:
-            ops.gemm_mid(logits, hidden_rows, w, mode=0)  # float32 sums, stored as they are
+            ops.gemm_mid(logits, hidden_rows, w, mode=0)
             return
-        low = ctx.buffers.get("head_logits_dt", S, self.vocab_size, hidden_rows.dtype,
-                              reserve=ctx.buffers.seq_capacity)
-        ops.linear(low, hidden_rows, w)
-        ops.to_float(logits, low)
+        ops.linear(logits, hidden_rows, w)  # the vendor product, float32 out
+
+
+OutputHead = LinearHead
+
+register_embedding("token_embedding", TokenEmbedding)
+register_head("linear_head", LinearHead)

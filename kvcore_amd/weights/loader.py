@@ -91,80 +91,78 @@ def load_weights(model: DecoderModel, model_dir: str | Path, *, strict: bool = T
 
 
 # ------------------------------------------------------------------- random weights
-_INIT_STD = {"normal": 0.02, "gain": 0.1}
+_INIT_RULES = {"normal": (0.0, 0.02), "gain": (1.0, 0.1)}  # (mean, standard deviation)
 
 
-def _tensor_seed(seed: int, name: str) -> int:
+def _tensor_seed(seed: int, name: str) -> tuple[int, int]:
+    """Two 32-bit words that key the generator for checkpoint tensor ``name``."""
     digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
-    return int.from_bytes(digest[:8], "little") & 0x7FFFFFFFFFFFFFFF
+    return int.from_bytes(digest[:4], "little"), int.from_bytes(digest[4:8], "little")
 
 
 def random_tensor(seed: int, name: str, shape: tuple[int, ...], init: str,
                   device: torch.device | str = "cpu") -> torch.Tensor:
-    """float32 values of checkpoint tensor ``name``: a function of (seed, name, device
-    kind) only, so they do not depend on the order in which tensors are made nor on how
-    they are stacked.  ``normal``: N(0, 0.02); ``gain``: 1 + N(0, 0.1); ``zeros``."""
+    """float32 values of checkpoint tensor ``name``: a function of (seed, name, element
+    index) only, so they depend neither on the order in which tensors are made, nor on how
+    they are stacked, nor on the device that draws them (the GPU kernel and its host twin,
+    ``weights/random_normal.py``, give the same bits).  ``normal``: N(0, 0.02); ``gain``:
+    1 + N(0, 0.1); ``zeros``."""
+    out = torch.empty(shape, dtype=torch.float32, device=device)
+    fill_random(out, seed, name, init)
+    return out
+
+
+def fill_random(out: torch.Tensor, seed: int, name: str, init: str) -> None:
+    """Fill the contiguous tensor ``out`` (float32 or bfloat16; bfloat16 receives the float32
+    values rounded to nearest even) with the values of checkpoint tensor ``name``."""
+    if not out.is_contiguous():
+        raise ValueError("fill_random needs a contiguous tensor")
     if init == "zeros":
-        return torch.zeros(shape, dtype=torch.float32, device=device)
-    gen = torch.Generator(device=device)
-    gen.manual_seed(_tensor_seed(seed, name))
-    t = torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * _INIT_STD[init]
-    if init == "gain":
-        t += 1.0
-    return t
+        out.zero_()
+        return
+    mean, std = _INIT_RULES[init]
+    lo, hi = _tensor_seed(seed, name)
+    if out.is_cuda:
+        from kvcore_amd.ops import library as ops
+
+        ops.fill_normal(out, lo, hi, mean, std)
+        return
+    from . import random_normal
+
+    values = torch.from_numpy(random_normal.normal(lo, hi, out.numel(), mean, std)).view(out.shape)
+    out.copy_(values)
 
 
-def init_random_weights(model: DecoderModel, seed: int, *, on_device: bool = True) -> None:
-    """Fill every parameter in place, checkpoint tensor by checkpoint tensor.  With
-    ``on_device`` the numbers are drawn on the GPU (fast for large models; they differ
-    from the CPU's draw of the same seed)."""
-    device = model.device if on_device else torch.device("cpu")
+def init_random_weights(model: DecoderModel, seed: int) -> None:
+    """Fill every parameter in place, checkpoint tensor by checkpoint tensor, on the model's
+    device: the same values that ``write_random_model`` stores for this seed (a matrix kept
+    in bfloat16 is the float32 draw rounded once, as a file of bfloat16 matrices holds it)."""
     for name, (bp, row, rows) in model.checkpoint_map().items():
-        shape = _expected_shape(bp, rows)
-        values = random_tensor(seed, name, shape, bp.spec.init, device)
-        bp.tensor.narrow(0, row, rows).copy_(values)
-        del values
+        fill_random(bp.tensor.narrow(0, row, rows), seed, name, bp.spec.init)
     if model.device.type == "cuda":
         torch.cuda.synchronize(model.device)
 
 
 def random_checkpoint_tensors(spec_params: dict[str, tuple[tuple[int, ...], str, str]], seed: int,
-                              dtype: torch.dtype) -> dict[str, torch.Tensor]:
+                              dtype: torch.dtype, device: torch.device | str = "cpu") -> dict[str, torch.Tensor]:
     """``{name: (shape, init, kind)}`` -> CPU tensors; matrices in ``dtype``, vectors in
-    float32."""
+    float32.  ``device`` is where the numbers are drawn (the values do not depend on it; a
+    GPU draws a large model far sooner)."""
     out = {}
     for name, (shape, init, kind) in spec_params.items():
-        t = random_tensor(seed, name, shape, init, "cpu")
-        out[name] = t.to(dtype) if kind == "matrix" else t
+        t = torch.empty(shape, dtype=dtype if kind == "matrix" else torch.float32, device=device)
+        fill_random(t, seed, name, init)
+        out[name] = t.cpu()
     return out
 
 
 def checkpoint_layout(model_spec) -> dict[str, tuple[tuple[int, ...], str, str]]:
     """The checkpoint tensors a model of this spec reads: name -> (shape, init rule,
     kind), derived from the parts' declarations without allocating the model."""
-    from kvcore_amd.parts import base as parts
-    from kvcore_amd.parts.embedding import OutputHead, TokenEmbedding
+    from kvcore_amd.models.decoder import build_parts
 
-    owned: list[tuple[str, parts.Part]] = [
-        (model_spec.embed_prefix, TokenEmbedding(vocab_size=model_spec.vocab_size,
-                                                 hidden_size=model_spec.hidden_size)),
-        (model_spec.final_norm_prefix, parts.NORMS.build(model_spec.final_norm)),
-        (model_spec.head_prefix, OutputHead(vocab_size=model_spec.vocab_size,
-                                            hidden_size=model_spec.hidden_size,
-                                            tied=model_spec.tie_word_embeddings)),
-    ]
-    for i, ps in enumerate(model_spec.positions):
-        prefix = model_spec.position_prefixes[i] if model_spec.position_prefixes else f"model.positions.{i}"
-        owned.append((prefix, parts.POSITION_ENCODINGS.build(ps)))
-    for layer in model_spec.layers:
-        mixer = parts.MIXERS.build(layer.mixer, position=None)
-        ffn = parts.FEED_FORWARDS.build(layer.ffn)
-        norms = {n: parts.NORMS.build(s) for n, s in layer.norms.items()}
-        block = parts.BLOCKS.build(layer.block, mixer=mixer, ffn=ffn, norms=norms)
-        for sub, part in block.children().items():
-            owned.append((f"{layer.prefix}.{sub}", part))
     layout: dict[str, tuple[tuple[int, ...], str, str]] = {}
-    for prefix, part in owned:
+    for prefix, part in build_parts(model_spec).owned:
         for ps in part.param_specs():
             for src in ps.resolved_sources():
                 layout[f"{prefix}.{src.name}"] = ((src.rows, *ps.shape[1:]), ps.init, ps.kind)
@@ -172,10 +170,11 @@ def checkpoint_layout(model_spec) -> dict[str, tuple[tuple[int, ...], str, str]]
 
 
 def write_random_model(folder: str | Path, config: dict, seed: int,
-                       dtype: torch.dtype = torch.bfloat16) -> Path:
+                       dtype: torch.dtype = torch.bfloat16, device: torch.device | str = "cpu") -> Path:
     """The random-weights mode as a folder: ``config.json`` and ``model.safetensors``
     made from a configuration mapping and a seed.  Matrices are stored in ``dtype``,
-    vectors (norm gains) in float32."""
+    vectors (norm gains) in float32.  ``device``: where the numbers are drawn, which does
+    not change them."""
     from kvcore_amd.registry import resolve_architecture
 
     arch = resolve_architecture(config)
@@ -183,7 +182,7 @@ def write_random_model(folder: str | Path, config: dict, seed: int,
     spec = arch.build_spec(typed)
     folder = Path(folder)
     folder.mkdir(parents=True, exist_ok=True)
-    tensors = random_checkpoint_tensors(checkpoint_layout(spec), seed, dtype)
+    tensors = random_checkpoint_tensors(checkpoint_layout(spec), seed, dtype, device)
     write_safetensors(folder / "model.safetensors", tensors, metadata={"format": "pt", "seed": str(seed)})
     (folder / "config.json").write_text(json.dumps(dict(config), indent=2) + "\n")
     return folder

@@ -99,15 +99,26 @@ def random_tokens(n: int, vocab: int, seed: int) -> list[int]:
 TINY_LOGIT_RMS = 0.2  # root mean square of the tiny models' logits (0.16 to 0.24)
 
 
-def tolerance(dtype: torch.dtype, logit_rms: float = TINY_LOGIT_RMS) -> dict:
+def tolerance(dtype: torch.dtype, logit_rms: float = TINY_LOGIT_RMS, sum_length: int = 0) -> dict:
     """Bounds on |engine - plain| for logits of the tiny models (|logit| is about 0.1 to
     1).  float32: both sides sum the same products in different orders, a few 1e-7
     relative per operation over a few hundred operations.  bfloat16: activations are
     rounded to 8 bits of mantissa (2^-9 relative) at about ten places per layer.
     The absolute part is 4% of the logits' root mean square (a small logit's error comes
-    from the large terms that cancel in it): a model with larger logits says so."""
+    from the large terms that cancel in it): a model with larger logits says so.
+
+    ``sum_length``: the longest sum of products in the model (its widest K), for models far
+    wider than the tiny ones.  A float32 sum of K terms taken in order errs, relative to its
+    result, in proportion to sqrt(K) (the rounding errors of the partial sums add up like a
+    random walk of steps that grow with the partial sums); the tiny models' sums have a few
+    hundred terms, so the float32 bound grows by sqrt(K / 1024) beyond 1024 terms (3.7 times
+    at the 14336 of Llama-3-8B's feed-forward; the worst error measured there, over 2e7
+    logits, is 0.3 of that bound, and a product in any reduced precision would miss it by a
+    factor of ten or more).  bfloat16 sums are float32 sums of products whose inputs were
+    rounded first: that rounding dominates whatever the length, so its bound stays."""
     scale = max(1.0, logit_rms / TINY_LOGIT_RMS)
     if dtype == torch.float32:
+        scale *= max(1.0, (sum_length / 1024) ** 0.5)
         return dict(atol=5e-6 * scale, rtol=2e-5)
     return dict(atol=8e-3 * scale, rtol=2e-2)
 

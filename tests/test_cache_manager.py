@@ -140,6 +140,45 @@ def test_two_groups_have_pages_of_their_own():
     m.check()
 
 
+def test_groups_are_planned_for_the_same_number_of_tokens():
+    from dataclasses import dataclass
+
+    from kvcore_amd.cache.kv_manager import plan_groups
+
+    @dataclass(frozen=True)
+    class Need:
+        page_size: int | None = None
+        window: int = 0
+
+    groups = plan_groups([Need(), Need(32, 0), Need(None, 64), Need(4, 0)], block_size=16, num_blocks=11)
+    assert [(g.page_size, g.num_pages, g.window) for g in groups] == [
+        (16, 11, 0), (32, 6, 0), (16, 11, 64), (4, 41, 0)]
+    for g in groups:  # each holds the 160 tokens that ten blocks of sixteen hold
+        assert (g.num_pages - 1) * g.page_size >= 160
+    with pytest.raises(ValueError):
+        plan_groups([Need()], 16, 1)
+
+
+def test_pages_given_back_are_logged_when_asked_for():
+    """The runner may poison pages that were given back; the manager says which they are."""
+    m = KVManager([GroupConfig(4, 10, 0), GroupConfig(4, 10, 8)], max_num_seqs=2, max_model_len=64,
+                  track_freed=True)
+    m.admit("r")
+    m.allocate("r", 0, 20)
+    assert m.drain_freed() == [[], []]
+    m.release_behind_window("r", 20)  # window 8: keys 13.. are needed, pages 0..2 go
+    assert m.drain_freed() == [[], [1, 2, 3]]
+    assert m.drain_freed() == [[], []]
+    m.free("r")
+    freed = m.drain_freed()
+    assert sorted(freed[0]) == [1, 2, 3, 4, 5] and sorted(freed[1]) == [4, 5]
+    quiet = make_manager()
+    quiet.admit("q")
+    quiet.allocate("q", 0, 4)
+    quiet.free("q")
+    assert quiet.drain_freed() == [[]]
+
+
 @pytest.mark.parametrize("seed", range(5))
 def test_no_page_is_lost_held_twice_or_freed_twice_under_random_traffic(seed):
     rng = random.Random(seed)

@@ -65,6 +65,24 @@ def test_eos_may_be_an_int_or_a_list():
     assert LlamaConfig.from_dict({**TINY_A, "eos_token_id": [7, 9]}).eos_token_ids == (7, 9)
 
 
+def test_generation_config_adds_stop_ids(tmp_path):
+    """An instruct checkpoint lists its end-of-turn id in generation_config.json only."""
+    import json
+
+    from kvcore_amd.config.model_config import ConfigError, read_generation_eos
+
+    assert read_generation_eos(tmp_path) == ()
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": [128001, 128009]}))
+    assert read_generation_eos(tmp_path) == (128001, 128009)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": 5, "temperature": 0.6}))
+    assert read_generation_eos(tmp_path) == (5,)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"temperature": 0.6}))
+    assert read_generation_eos(tmp_path) == ()
+    (tmp_path / "generation_config.json").write_text("{not json")
+    with pytest.raises(ConfigError):
+        read_generation_eos(tmp_path)
+
+
 def test_registry_key_is_the_architecture_name_with_model_type_as_fallback():
     assert resolve_architecture(TINY_A).name == "LlamaForCausalLM"
     assert resolve_architecture({"model_type": "llama"}).name == "LlamaForCausalLM"

@@ -65,8 +65,8 @@ def collect(session, steps):
     return got
 
 
-def compare(got, expect_by_id, dtype, logit_rms=None):
-    tol = tolerance(dtype) if logit_rms is None else tolerance(dtype, logit_rms)
+def compare(got, expect_by_id, dtype, logit_rms=None, sum_length=0):
+    tol = tolerance(dtype, sum_length=sum_length) if logit_rms is None else tolerance(dtype, logit_rms, sum_length)
     assert got, "nothing was compared"
     from tests import helpers
     for (rid, pos), row in sorted(got.items()):
@@ -259,6 +259,60 @@ def test_logits_do_not_depend_on_which_pages_are_used(models, dtype):
     assert results[0].keys() == results[1].keys()
     for key, row in results[0].items():
         assert torch.equal(row, results[1][key]), key
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_float32_logits_are_the_same_bits_under_every_cut(models, name):
+    """In float32 every product element is one sum in k order, a token's attention depends on
+    its position alone and norms work row by row: so the logits at a (request, position) must
+    not differ by a single bit between a whole prompt, tokens one by one, portions of changing
+    size and mixed batches on reused pages."""
+    folder, cfg, weights, page = models[name]
+    base = PROMPT_LENS[name]
+    lens = base + [base[-1] + 17, base[0] + 1]
+    token_lists = {f"q{i}": random_tokens(n + EXTRA, cfg["vocab_size"], seed=900 + i) for i, n in enumerate(lens)}
+    whole = {}
+    for rid, tokens in token_lists.items():
+        session = session_for(folder, torch.float32, page, max_tokens=len(tokens))
+        whole.update(collect(session, [{"step": 0, "entries": [
+            {"id": rid, "tokens": tokens, "want": list(range(len(tokens)))}], "end": [rid]}]))
+    compared = 0
+
+    def same(got, what):
+        nonlocal compared
+        for key, row in got.items():
+            assert torch.equal(row, whole[key]), f"{what}: {key} differs from the whole prompt by " \
+                                                 f"{float((row - whole[key]).abs().max()):.3e}"
+            compared += 1
+
+    sizes = [16, 7, 2, 5, 13, 2, 3, 9, 2, 11, 4, 2]
+    for rid, tokens in token_lists.items():
+        # most of it in one step, the last 32 tokens one by one
+        head = len(tokens) - 32
+        session = session_for(folder, torch.float32, page, max_tokens=len(tokens))
+        steps = [{"step": 0, "entries": [{"id": rid, "tokens": tokens[:head], "want": [head - 1]}], "end": []}]
+        steps += [{"step": j + 1, "entries": [{"id": rid, "tokens": [tokens[head + j]], "want": [0]}], "end": []}
+                  for j in range(32)]
+        same(collect(session, steps), "one by one")
+        # portions of changing size
+        session = session_for(folder, torch.float32, page, max_tokens=len(tokens))
+        steps, at, k = [], 0, 0
+        while at < len(tokens):
+            size = min(sizes[k % len(sizes)], len(tokens) - at)
+            if len(tokens) - at - size == 1:
+                size += 1
+            steps.append({"step": k, "entries": [{"id": rid, "tokens": tokens[at:at + size],
+                                                  "want": list(range(size))}], "end": []})
+            at += size
+            k += 1
+        same(collect(session, steps), "portions")
+    # mixed, with so few pages that they are used again
+    rounded = sorted((-(-len(t) // 64) * 64 for t in token_lists.values()), reverse=True)
+    session = session_for(folder, torch.float32, page, max_tokens=sum(rounded[:4]))
+    got = collect(session, mixed_trace(token_lists, seed=12))
+    assert len(got) == sum(len(t) for t in token_lists.values())
+    same(got, "mixed")
+    assert compared > 3 * len(got) // 2
 
 
 def collect_one(session, rec, starts):

@@ -281,3 +281,88 @@ def test_chat_messages_in_and_text_out(folders, tmp_path):
     # a request without a tokenizer-made prompt needs token ids
     with pytest.raises(ValueError):
         engine.generate([GenerationRequest("bad", SamplingParams(max_tokens=2))])
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 5e-5), ("bfloat16", 6e-2)])
+def test_preemption_with_seeded_sampling_and_steps_launched_ahead(folders, dtype, tol):
+    """So few pages that running requests are preempted and recomputed, with seeded
+    temperature sampling, in both dtypes, with and without steps launched ahead: a preempted
+    request's noise stream goes on where it was (nothing is drawn twice), every token is the
+    plain sampler's choice on the plain logits, and launching ahead changes no token."""
+    from kvcore_amd import SamplingParams
+
+    folder, cfg, weights, page = folders["A"]
+    prompts = {f"r{i}": random_tokens(n, 256, seed=320 + i) for i, n in enumerate((20, 30, 25, 18))}
+    reqs = [dict(request_id=rid, prompt_token_ids=p,
+                 sampling_params=SamplingParams(max_tokens=30, temperature=0.8, seed=900 + i, ignore_eos=True))
+            for i, (rid, p) in enumerate(prompts.items())]
+    results = {}
+    for run_ahead in (False, True):
+        tight = make_engine(folder, dtype, page, num_pages=9, run_ahead=run_ahead)  # 8 usable pages
+        results[run_ahead] = {o.request_id: o.output_token_ids for o in tight.generate(reqs)}
+        assert tight.engine_core.scheduler.num_preemptions > 0
+        assert tight.engine_core.kv_manager.num_free_pages() == [8]
+    assert results[True] == results[False]
+    for i, (rid, p) in enumerate(prompts.items()):
+        toks = results[True][rid]
+        assert len(toks) == 30
+        check_tokens(cfg, weights, p, toks, temperature=0.8, seed=900 + i, tol=tol)
+    if dtype == "float32":  # and they are the tokens of an engine that never ran out of pages
+        roomy = make_engine(folder, dtype, page)
+        assert {o.request_id: o.output_token_ids for o in roomy.generate(reqs)} == results[True]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_engine_equals_a_replay_of_the_trace_its_scheduler_produced(folders, dtype):
+    """Every step the engine runs is recorded as a trace step (request, tokens, wanted places,
+    requests that ended) and fed again through the replay session, which has neither
+    scheduler nor sampler: the logits of every step must be the engine's (in float32 bit for
+    bit, wherever the replay's pages lie)."""
+    from kvcore_amd import SamplingParams
+    from kvcore_amd.engine.replay import TraceSession
+
+    folder, cfg, weights, page = folders["B"]
+    prompts = {f"r{n}": random_tokens(n, 384, seed=600 + n) for n in (1, 9, 24, 40, 61)}
+    core = make_engine(folder, dtype, page, budget=24, threshold=16, max_seqs=3, run_ahead=False).engine_core
+    steps: list[tuple[list, torch.Tensor | None]] = []
+    real_step = core.runner.step
+
+    def recording_step(entries, device_tokens=None):
+        out = real_step(entries, device_tokens)
+        steps.append(([(e.request_id, list(e.tokens), list(e.want)) for e in entries],
+                      None if out.logits is None else out.logits.clone()))
+        return out
+
+    core.runner.step = recording_step
+    for i, (rid, p) in enumerate(prompts.items()):
+        if i < 4:
+            core.add_request(rid, SamplingParams(max_tokens=12 + i, temperature=0.7, seed=50 + i, ignore_eos=True),
+                             prompt_token_ids=p)
+    ends: list[list[str]] = []
+    while core.has_unfinished_requests():
+        before = len(steps)
+        outs = core.step()
+        assert len(steps) == before + 1
+        ends.append([o.request_id for o in outs.request_outputs if o.finished])
+        if len(steps) == 5:  # a late arrival
+            core.add_request("r61", SamplingParams(max_tokens=9, temperature=0.0, ignore_eos=True),
+                             prompt_token_ids=prompts["r61"])
+    assert any(len(entries) > 1 and any(len(t) > 1 for _, t, _ in entries) and any(len(t) == 1 for _, t, _ in entries)
+               for entries, _ in steps), "some step should mix a portion of a prompt with decoded tokens"
+    session = TraceSession(str(folder), getattr(torch, dtype), max_tokens=3 * 128, block_size=page,
+                           poison_cache=True, shuffle_pages=5)
+    compared = 0
+    for k, ((entries, logits), end) in enumerate(zip(steps, ends)):
+        out = session.run_step({"step": k, "end": end, "entries": [
+            {"id": rid, "tokens": tokens, "want": want} for rid, tokens, want in entries]})
+        if logits is None:
+            assert out.logits is None
+            continue
+        assert out.logits.shape == logits.shape
+        if dtype == "float32":
+            assert torch.equal(out.logits, logits), f"step {k}"
+        else:  # the replay plans its launches for another length limit: rounding may differ
+            assert torch.allclose(out.logits, logits, atol=2e-2, rtol=2e-2), f"step {k}"
+        compared += logits.shape[0]
+    assert compared >= sum(12 + i for i in range(4)) + 9
+    assert session.manager.live_requests() == []

@@ -43,6 +43,8 @@ def test_embed(ops, dtype):
     ops.embed(out, table, ids)
     assert torch.equal(out[:4], table.float()[ids[:4].long()])
     assert torch.isnan(out[4:]).all()  # an id outside the table is loud, not a stray read
+    ops.embed(out, table, ids, 2.5)
+    assert torch.equal(out[:4], table.float()[ids[:4].long()] * 2.5)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -382,17 +384,102 @@ def test_linear_picks_a_kernel_by_row_count(ops):
         out = torch.empty(M, 96, dtype=torch.bfloat16, device=DEV)
         ops.linear(out, x, w)
         assert torch.allclose(out.double(), x.double() @ w.double().T, atol=2e-2, rtol=2e-2)
-    with pytest.raises(ops.KernelError):
-        ops.linear(torch.empty(100, 96, device=DEV), rnd(100, 256, dtype=torch.bfloat16), w)
+    # a float32 result keeps the float32 sums unrounded on every path (few rows: our kernel;
+    # more: the vendor product asked for float32)
+    bias = rnd(96, dtype=torch.bfloat16, seed=9)
+    for M in (3, 12, 40, 100, 200):
+        x = rnd(M, 256, dtype=torch.bfloat16, seed=M)
+        for b in (None, bias):
+            out = torch.empty(M, 96, device=DEV)
+            ops.linear(out, x, w, b)
+            want = x.double() @ w.double().T + (0 if b is None else b.double())
+            assert torch.allclose(out.double(), want, atol=2e-6, rtol=2e-6), (M, b is not None)
 
 
-def test_bf16_linear_uses_float32_accumulation(ops):
-    x, w = rnd(5, 300, dtype=torch.bfloat16), rnd(70, 300, dtype=torch.bfloat16)
-    bias = rnd(70, dtype=torch.bfloat16)
-    out = torch.empty(5, 70, dtype=torch.bfloat16, device=DEV)
-    ops.linear(out, x, w, bias)
-    want = x.double() @ w.double().T + bias.double()
-    assert torch.allclose(out.double(), want, atol=0.15, rtol=1e-2)
+@pytest.mark.parametrize("M", [5, 12, 40, 100])
+def test_bf16_products_sum_in_float32(ops, M):
+    """Inputs of one sign and a long K: every product is 1 + 2^-7 exactly and every partial sum
+    is a multiple of 2^-7 below 2^24, so float32 sums are exact in any order (4128), while a
+    sum kept in bfloat16 would stall at 256."""
+    K, N = 4096, 128
+    x = torch.ones(M, K, dtype=torch.bfloat16, device=DEV)
+    w = torch.full((N, K), 1.0 + 2.0 ** -7, dtype=torch.bfloat16, device=DEV)
+    want = torch.full((M, N), 4096 * (1.0 + 2.0 ** -7), device=DEV)
+    out = torch.empty(M, N, device=DEV)
+    ops.linear(out, x, w)
+    assert torch.equal(out, want)
+    out16 = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(out16, x, w)
+    assert torch.equal(out16.float(), want.to(torch.bfloat16).float())  # rounded once, at the end
+    if M <= ops.SKINNY_MAX_ROWS:
+        out.zero_()
+        ops.gemm_skinny_bf16(out, x, w)
+        assert torch.equal(out, want)
+        out.zero_()
+        ops.gemm_mid(out, x, w, mode=0)
+        assert torch.equal(out, want)
+
+
+def test_logits_finish_bias_cap_and_scale(ops):
+    """kvcore/sample/logits_processor.py:44-54: bias, then the soft cap, then the scale; the
+    reference's own vector (tests/test_sampler.py:20-26): logits [2, -2] under a cap of 1
+    stay within [-1, 1]."""
+    logits = torch.tensor([[2.0, -2.0]], device=DEV)
+    ops.logits_finish(logits, None, 1.0, 1.0)
+    assert torch.allclose(logits.cpu(), torch.tanh(torch.tensor([[2.0, -2.0]])), atol=1e-6)
+    assert (logits.abs() <= 1.0).all()
+    x = rnd(7, 1001, seed=3, scale=3.0)
+    wide = torch.zeros(7, 1100, device=DEV)
+    wide[:, :1001] = x
+    for bias in (None, rnd(1001, dtype=torch.bfloat16, seed=4), rnd(1001, seed=5)):
+        got = wide.clone()
+        ops.logits_finish(got[:, :1001], bias, 2.5, 0.5)
+        want = x.double() + (0 if bias is None else bias.double())
+        want = torch.tanh(want / 2.5) * 2.5 * 0.5
+        assert torch.allclose(got[:, :1001].double(), want, atol=1e-6)
+        assert (got[:, 1001:] == 0).all()
+    plainly = x.clone()
+    ops.logits_finish(plainly, None, 0.0, 1.0)
+    assert torch.equal(plainly, x)
+
+
+def test_fill_pages_touches_the_listed_pages_only(ops):
+    for dtype in DTYPES:
+        kv = torch.zeros(3, 2, 9, 2, 4, 16, dtype=dtype, device=DEV)  # [planes, k/v, pages, heads, page, d]
+        triples = torch.tensor([0, 0, 4, 1, 1, 0, 0, 1, 7, 2, 0, 99], dtype=torch.int32, device=DEV)
+        ops.fill_pages(kv, triples[2:], 4, float("nan"), stride=3)  # pages 4, 0 (null), 7, 99 (outside)
+        nan_pages = torch.isnan(kv.float()).flatten(3).all(dim=3)     # [3, 2, 9]
+        any_nan = torch.isnan(kv.float()).flatten(3).any(dim=3)
+        assert nan_pages[:, :, [4, 7]].all()
+        assert not any_nan[:, :, [0, 1, 2, 3, 5, 6, 8]].any()
+        pages = torch.tensor([1, 8], dtype=torch.int32, device=DEV)
+        ops.fill_pages(kv, pages, 2, 0.5)
+        assert (kv[:, :, [1, 8]] == 0.5).all() and (kv[:, :, 2] == 0).all()
+
+
+def test_random_fill_gives_the_host_generator_bits(ops):
+    """The kernel and its host twin draw the same values for one seed, in float32 and rounded
+    to bfloat16, so a model drawn on the GPU is the model that a written folder holds."""
+    import numpy as np
+
+    from kvcore_amd.weights import random_normal
+
+    n = 3_000_017  # covers every table entry and both tails many times over
+    for lo, hi, mean, std in ((123, 456, 0.0, 0.02), (0xFFFFFFFF, 7, 1.0, 0.1)):
+        want = torch.from_numpy(random_normal.normal(lo, hi, n, mean, std))
+        got = torch.empty(n, device=DEV)
+        ops.fill_normal(got, lo, hi, mean, std)
+        assert torch.equal(got.cpu().view(torch.int32), want.view(torch.int32))
+        got16 = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+        ops.fill_normal(got16, lo, hi, mean, std)
+        assert torch.equal(got16.cpu().view(torch.int16), want.to(torch.bfloat16).view(torch.int16))
+    z = (want.double() - 1.0) / 0.1
+    assert abs(float(z.mean())) < 3e-3 and abs(float(z.std()) - 1.0) < 3e-3
+    assert 4.5 < float(z.abs().max()) < 6.5
+    # an index beyond 32 bits changes the draw (the high word is mixed in)
+    a = random_normal.standard_normal(1, 2, 5, 4)
+    b = random_normal.standard_normal(1, 2, 5 + (1 << 32), 4)
+    assert not np.array_equal(a, b)
 
 
 def test_rope_table(ops):

@@ -207,3 +207,74 @@ def test_prenorm_block_against_the_reference_arrangement():
     assert torch.allclose(residual.double().cpu(), r2, atol=1e-5)
     with pytest.raises(ValueError, match="norms"):
         BLOCKS.build(PartSpec("prenorm"), mixer=Doubler(), ffn=Negate(), norms={})
+
+
+def test_head_part_scale_vector_of_the_reference():
+    """tests/test_sampler.py:10-17 of the reference: weight [[1,0],[0,1],[1,1]], hidden [2,3],
+    scale 0.5 give [1.0, 1.5, 2.5], through the head part itself."""
+    from kvcore_amd.parts.base import HEADS, PartSpec, Runtime
+
+    for dtype in DTYPES:
+        head = HEADS.build(PartSpec("linear_head", {"vocab_size": 3, "hidden_size": 2, "logit_scale": 0.5}))
+        head.setup(Runtime(dtype, DEV))
+        head.bind({"weight": torch.tensor([[1.0, 0.0], [0.0, 1.0], [1.0, 1.0]], dtype=dtype, device=DEV)})
+        logits = torch.empty(1, 3, device=DEV)
+        head.forward(logits, torch.tensor([[2.0, 3.0]], dtype=dtype, device=DEV), make_ctx(dtype, [0], [0], [0]))
+        assert torch.equal(logits.cpu(), torch.tensor([[1.0, 1.5, 2.5]]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [3, 14, 40, 70])
+def test_head_part_keeps_float32_sums_whatever_the_row_count(dtype, rows):
+    """A vocabulary beyond 65536 entries sends 3, 14, 40 and 70 rows down the head's four
+    branches; all of them store the float32 sums unrounded (a row's logits must not change
+    their rounding with the rows beside it), with bias, soft cap and scale applied after."""
+    from kvcore_amd.parts.base import HEADS, PartSpec
+
+    V, H = 70016, 512
+    head = HEADS.build(PartSpec("linear_head", {"vocab_size": V, "hidden_size": H, "bias": True,
+                                                 "soft_cap": 30.0, "logit_scale": 0.25}))
+    p = bind_random(head, dtype, seed=rows)
+    bias = (torch.randn(V, generator=torch.Generator().manual_seed(1)) * 0.3).to(dtype).to(DEV)
+    head.bind({**head.params, "bias": bias})
+    x = (torch.randn(rows, H, generator=torch.Generator().manual_seed(2))).to(dtype).to(DEV)
+    logits = torch.empty(rows, V, device=DEV)
+    head.forward(logits, x, make_ctx(dtype, [0] * rows, list(range(rows)), list(range(rows))))
+    want = x.double().cpu() @ p["weight"].T + bias.double().cpu()
+    want = torch.tanh(want / 30.0) * 30.0 * 0.25
+    # the operands are the same bits on both sides, so only the order of the float32 sums differs
+    assert torch.allclose(logits.double().cpu(), want, atol=2e-5, rtol=1e-5)
+    # and the first rows alone give the bits they had in company
+    alone = torch.empty(2, V, device=DEV)
+    head.forward(alone, x[:2].contiguous(), make_ctx(dtype, [0, 0], [0, 1], [0, 1]))
+    assert torch.allclose(alone, logits[:2], atol=2e-5, rtol=1e-5)
+
+
+def test_embedding_part_scale():
+    from kvcore_amd.parts.base import EMBEDDINGS, PartSpec
+
+    for dtype in DTYPES:
+        emb = EMBEDDINGS.build(PartSpec("token_embedding", {"vocab_size": 50, "hidden_size": 24, "scale": 3.0}))
+        p = bind_random(emb, dtype)
+        ids = torch.tensor([4, 49, 0], dtype=torch.int32, device=DEV)
+        out = torch.empty(3, 24, device=DEV)
+        emb.forward(out, ids)
+        assert torch.allclose(out.double().cpu(), p["weight"][ids.long().cpu()] * 3.0, atol=1e-6)
+
+
+def test_attention_refuses_a_block_table_wider_than_its_decode_kernel_serves():
+    """At construction of a runner, not in the middle of a generation."""
+    from kvcore_amd.ops import library as ops
+    from kvcore_amd.parts.base import MIXERS, PartSpec, RunLimits, Runtime
+
+    attn = MIXERS.build(PartSpec("paged_attention", {"hidden_size": 4096, "num_heads": 32, "num_kv_heads": 8,
+                                                     "head_dim": 128, "scale": 128 ** -0.5}), position=None)
+    attn.setup(Runtime(torch.bfloat16, DEV))
+    widest = ops.decode_attention_max_table(32, 8, 128)
+    assert widest >= 8192  # 131,072 tokens in pages of 16
+    attn.check_limits(RunLimits(8, 512, widest * 16, 16, widest))
+    with pytest.raises(ValueError, match="block_size"):
+        attn.check_limits(RunLimits(8, 512, (widest + 1) * 16, 16, widest + 1))
+    # float32 runs the general kernel, which has no such limit
+    attn.setup(Runtime(torch.float32, DEV))
+    attn.check_limits(RunLimits(8, 512, (widest + 1) * 16, 16, widest + 1))

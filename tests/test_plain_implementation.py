@@ -100,6 +100,52 @@ def test_llama3_scaling_bands():
     assert (out[1:] < out[:-1]).all()
 
 
+def test_llama3_blend_is_continuous_at_both_band_edges_and_hits_a_hand_worked_value():
+    """What pins the blend's direction.  At a wavelength just inside the middle band next to
+    the short-wave edge (``original / high``) the result must meet the kept frequency, and
+    next to the long-wave edge (``original / low``) the divided one; a blend with ``s`` and
+    ``1 - s`` exchanged jumps by a factor of ``factor`` at both.  And config B's one blended
+    index, worked by hand from the rule of the config keys: d = 32, theta = 5e5, index 2:
+    ln 5e5 = 13.1223634, so inv_freq = exp(-13.1223634 / 8) = 0.193923, wavelength 2 pi /
+    inv_freq = 32.4004, original / wavelength = 64 / 32.4004 = 1.975284, s = (1.975284 - 1) /
+    (4 - 1) = 0.325095, (1 - s) / 8 + s = 0.084363 + 0.325095 = 0.409458 (with s and 1 - s
+    exchanged it would be 0.715542)."""
+    from kvcore_amd.parts.rotary import rotary_inv_freq
+
+    kw = dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=64)
+    inv = plain.rope_inv_freq(32, 500000.0)
+    out = plain.llama3_scale_inv_freq(inv, **kw)
+    assert float(out[2] / inv[2]) == pytest.approx(0.409458, abs=5e-6)
+    product = rotary_inv_freq(32, 500000.0, {"rope_type": "llama3", **kw})
+    assert float(product[2]) / float(inv[2]) == pytest.approx(0.409458, abs=5e-6)
+
+    def scaled(wavelen):
+        f = torch.tensor([2 * math.pi / wavelen], dtype=torch.float64)
+        return float(plain.llama3_scale_inv_freq(f, **kw)[0]), float(f[0])
+
+    short_edge, long_edge = 64 / 4.0, 64 / 1.0
+    got, f = scaled(short_edge * (1 + 1e-9))   # just inside the middle band
+    assert got == pytest.approx(f, rel=1e-6)   # meets the band that is kept
+    got, f = scaled(short_edge * (1 - 1e-9))
+    assert got == f
+    got, f = scaled(long_edge * (1 - 1e-9))    # just inside the middle band
+    assert got == pytest.approx(f / 8.0, rel=1e-6)  # meets the band that is divided
+    got, f = scaled(long_edge * (1 + 1e-9))
+    assert got == pytest.approx(f / 8.0, rel=1e-12)
+    # the middle of the band in original / wavelength (2.5 of 1..4) is the mean of both
+    got, f = scaled(64 / 2.5)
+    assert got == pytest.approx(0.5 * (f + f / 8.0), rel=1e-12)
+    # the product's own table follows the same rule at the sizes of the large models
+    for d, theta, factor in ((128, 500000.0, 8.0), (64, 500000.0, 32.0)):
+        big = dict(factor=factor, low_freq_factor=1.0, high_freq_factor=4.0,
+                   original_max_position_embeddings=8192)
+        want = plain.llama3_scale_inv_freq(plain.rope_inv_freq(d, theta), **big)
+        have = rotary_inv_freq(d, theta, {"rope_type": "llama3", **big})
+        assert torch.allclose(have.double(), want, rtol=1e-6)
+        wl = 2 * math.pi / plain.rope_inv_freq(d, theta)
+        assert ((wl >= 8192 / 4) & (wl <= 8192)).sum() >= 3, "some indices are blended at these sizes"
+
+
 # ------------------------------------------------------------------------- attention
 def test_attention_equals_library_causal_attention():
     T, nh, nkv, d = 9, 6, 2, 16
@@ -253,12 +299,6 @@ def test_layer_order_matches_the_carried_residual_form():
 
 
 # -------------------------------------------------------------------------- sampling
-def test_head_scale_vector_of_the_reference():
-    """tests/test_sampler.py:10-17: weight [[1,0],[0,1],[1,1]], hidden [2,3], scale 0.5."""
-    w = torch.tensor([[1.0, 0.0], [0.0, 1.0], [1.0, 1.0]])
-    assert torch.allclose((torch.tensor([[2.0, 3.0]]) @ w.T) * 0.5, torch.tensor([[1.0, 1.5, 2.5]]))
-
-
 def test_greedy_vectors_of_the_reference():
     """tests/test_sampler.py:29-35."""
     assert plain_sampling.sample(torch.tensor([0.0, 2.0, 1.0]), temperature=0.0) == 1

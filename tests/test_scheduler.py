@@ -180,6 +180,51 @@ def test_when_pages_run_out_the_last_admitted_request_is_preempted_and_recompute
     assert s.kv_manager.num_free_pages() == [6]
 
 
+def test_a_request_that_recomputes_after_preemption_counts_as_a_prefill():
+    """After a preemption the prompt and the output so far are computed again as one prompt;
+    while that lasts the request counts against ``max_num_partial_prefills`` (and, by its new
+    length, against the limit on long ones), also beyond its original prompt's length."""
+    cfg = SchedulerConfig(max_num_seqs=3, max_num_scheduled_tokens=3, max_num_partial_prefills=1,
+                          long_prefill_token_threshold=0)
+    s = make_scheduler(cfg, num_pages=40, page=2, max_len=32)
+    victim = make_request("victim", [1, 2], max_tokens=12)
+    s.add_request(victim)
+    for token in range(6):  # prompt, then five decode steps: 2 + 6 tokens known
+        out = s.schedule()
+        s.update_from_outputs(out, {"victim": 50 + token})
+    assert victim.num_tokens == 8 and not s._is_prefill(victim)
+    s._preempt(victim)
+    assert victim.num_prefill_tokens == 8 and s._is_prefill(victim)
+    s.add_request(make_request("other", [7, 8, 9, 10], max_tokens=2))
+    out = s.schedule()  # budget 3: the victim recomputes tokens 0..2 and is the one prefill
+    assert out.num_scheduled_tokens == {"victim": 3}
+    s.update_from_outputs(out, {})
+    out = s.schedule()  # past its prompt's two tokens, it is still the one prefill allowed
+    assert victim.num_computed_tokens == 3 and s._is_prefill(victim)
+    assert out.num_scheduled_tokens == {"victim": 3}
+    s.update_from_outputs(out, {})
+    out = s.schedule()
+    assert out.num_scheduled_tokens == {"victim": 2} and shares(out)["victim"].samples
+    s.update_from_outputs(out, {"victim": 99})
+    assert not s._is_prefill(victim)
+    out = s.schedule()  # now it decodes, and the other request may start its prompt
+    assert out.num_scheduled_tokens == {"victim": 1, "other": 2}
+    # a long recomputation is a long prefill
+    cfg = SchedulerConfig(max_num_seqs=3, max_num_scheduled_tokens=16, max_num_partial_prefills=3,
+                          max_long_partial_prefills=1, long_prefill_token_threshold=4)
+    s = make_scheduler(cfg, num_pages=40, page=2, max_len=32)
+    victim = make_request("victim", [1, 2], max_tokens=12)
+    s.add_request(victim)
+    for token in range(5):
+        s.update_from_outputs(s.schedule(), {"victim": 50 + token})
+    assert not s._is_long_prefill(victim)
+    s._preempt(victim)
+    assert s._is_long_prefill(victim)
+    s.add_request(make_request("long", list(range(6)), max_tokens=1))
+    out = s.schedule()
+    assert out.num_scheduled_tokens == {"victim": 4}  # one long prefill at a time
+
+
 def test_no_progress_is_reported_when_nothing_can_run():
     cfg = SchedulerConfig(max_num_seqs=1, max_num_scheduled_tokens=4)
     s = make_scheduler(cfg, num_pages=4, page=2, max_len=6)

@@ -54,6 +54,45 @@ def test_random_weights_mode_is_a_function_of_seed_and_name(tmp_path):
         str(write_random_model(tmp_path / "t", TINY_B, seed=1) / "model.safetensors"))  # tied
 
 
+def test_random_values_depend_on_seed_name_and_index_only():
+    """Not on how the draw is cut into chunks, not on the tensor's shape or on what it is
+    stacked with; the kernel's tables are the ones worked out here."""
+    import math
+    import re
+    from pathlib import Path
+
+    import numpy as np
+
+    from kvcore_amd.weights import random_normal
+    from kvcore_amd.weights.loader import random_tensor
+
+    whole = random_normal.normal(11, 22, 100_000, 0.0, 0.02)
+    for chunk in (1, 7, 4096, 1 << 20):
+        n = 1000 if chunk < 100 else 100_000
+        assert np.array_equal(random_normal.normal(11, 22, n, 0.0, 0.02, chunk=chunk), whole[:n])
+    assert np.array_equal(random_normal.standard_normal(11, 22, 500, 100) * np.float32(0.02), whole[500:600])
+    a = random_tensor(3, "model.layers.0.self_attn.k_proj.weight", (8, 16), "normal")
+    b = random_tensor(3, "model.layers.0.self_attn.k_proj.weight", (4, 32), "normal")
+    assert torch.equal(a.flatten(), b.flatten())
+    assert not torch.equal(a, random_tensor(3, "model.layers.0.self_attn.v_proj.weight", (8, 16), "normal"))
+    assert not torch.equal(a, random_tensor(4, "model.layers.0.self_attn.k_proj.weight", (8, 16), "normal"))
+    gain = random_tensor(3, "model.norm.weight", (4096,), "gain")
+    assert abs(float(gain.mean()) - 1.0) < 0.01 and abs(float(gain.std()) - 0.1) < 0.01
+    assert (random_tensor(3, "x.bias", (5,), "zeros") == 0).all()
+    # the distribution: mean, deviation, tails and a Kolmogorov-Smirnov distance
+    z = np.sort(random_normal.standard_normal(5, 6, 0, 400_000).astype(np.float64))
+    assert abs(z.mean()) < 5e-3 and abs(z.std() - 1.0) < 5e-3
+    cdf = 0.5 * (1.0 + np.vectorize(math.erf)(z[::40] / math.sqrt(2.0)))
+    assert np.abs(cdf - (np.arange(0, 400_000, 40) + 0.5) / 400_000).max() < 4e-3
+    assert abs((np.abs(z) > 3).mean() - 0.0027) < 5e-4
+    # the kernel's source holds the same two tables, bit for bit
+    src = (Path(random_normal.__file__).resolve().parents[1] / "csrc" / "random_fill.hip").read_text()
+    for name, table in (("kInvC", random_normal.INV_C), ("kLnC", random_normal.LN_C)):
+        body = src[src.index(name + "[32]"):]
+        body = body[:body.index("};")]
+        assert [int(h, 16) for h in re.findall(r"0x([0-9A-F]{8})u", body)] == table.view(np.uint32).tolist()
+
+
 def checkpoint_layout_names(config):
     from kvcore_amd.registry import resolve_architecture
 
