@@ -8,10 +8,18 @@ batch 8 from 512-token prompts, context limit 8192.  One JSON line is printed:
 ``roofline`` prices the decode step's mandatory reads (every weight once, the live
 requests' cache) against 8 TB/s; ``points`` holds decode at batch 1 and 64.
 
+Before anything is timed, the tokens are checked (``check`` in the line): one request runs
+a short prompt and eight greedy decode steps through the step function; its logits must be
+finite, its tokens inside the vocabulary, and every token must be the plain implementation's
+choice (``tests/plain``, float32 on the CPU, the same weights) or tie with it within the
+rounding noise of bfloat16.  ``--check basic`` leaves the plain implementation out,
+``--check none`` all of it; the 70b shape only runs the basic check.
+
 Other workloads print a line of their own: ``--only-prefill``, ``--mixed`` (64 requests
 with prompts of 16 to 2,048 tokens in portions of 512), ``--long-prompt N`` (time to the
-first token of one N-token prompt in portions of 2,048); ``--model 1b|70b`` and ``--batch``
-change the shape.
+first token of one N-token prompt in portions of 2,048), ``--sweep`` (decode at further
+batch sizes and context lengths, a line each with its share of the memory bandwidth);
+``--model 1b|70b`` and ``--batch`` change the shape.
 """
 
 from __future__ import annotations
@@ -77,7 +85,77 @@ def parse_args():
     p.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     p.add_argument("--only-prefill", action="store_true",
                    help="run only the 2,048-token prefill (for profiling); prints its own line")
+    p.add_argument("--check", default=None, choices=["plain", "basic", "none"],
+                   help="check the tokens before timing: against the plain implementation on the CPU "
+                        "(default for the 8b and 1b shapes), finite logits and tokens in range only, "
+                        "or not at all")
+    p.add_argument("--sweep", action="store_true",
+                   help="instead of the default run: decode at batch 1..64 and at contexts of 8k, 32k "
+                        "and 128k tokens, a line each")
     return p.parse_args()
+
+
+def check_tokens(engine, cfg, mode, dtype_name):
+    """A short prompt and eight greedy decode steps through the engine's own step function and
+    cache; returns the record for the result line, raises if the tokens are not right."""
+    import torch
+
+    from kvcore_amd.engine.runner import StepEntry
+
+    rng = random.Random(7)
+    vocab = cfg["vocab_size"]
+    prompt = [rng.randrange(vocab) for _ in range(40)]
+    manager, runner = engine.kv_manager, engine.runner
+    rid = "bench-check"
+    manager.admit(rid)
+    slot = manager.slot_of(rid)
+    runner.forget(slot)
+    tokens, rows = [], []
+    ids, start = list(prompt), 0
+    for step in range(9):  # the prompt, then eight single tokens (the second is captured as a graph)
+        assert manager.allocate(rid, start, len(ids)) is not None
+        out = runner.step([StepEntry(rid, slot, start, ids, manager.page_ids(rid), (len(ids) - 1,),
+                                     manager.released_counts(rid))])
+        row = out.logits[0].float().cpu()
+        if not bool(torch.isfinite(row).all()):
+            raise RuntimeError(f"bench check: step {step} gave logits that are not finite")
+        tok = int(row.argmax())
+        if not 0 <= tok < vocab:
+            raise RuntimeError(f"bench check: token {tok} outside the vocabulary")
+        rows.append(row)
+        tokens.append(tok)
+        start += len(ids)
+        ids = [tok]
+    runner.forget(slot)
+    manager.free(rid)
+    record = {"tokens": len(tokens), "finite": True, "in_range": True}
+    if mode != "plain":
+        return record
+    from tests.plain import llama as plain
+
+    t0 = time.perf_counter()
+    weights = {}
+    for name, (bp, row, nrows) in engine.model.checkpoint_map().items():
+        weights[name] = bp.tensor.narrow(0, row, nrows).float().cpu()
+    sequence = prompt + tokens[:-1]
+    logits = plain.llama_forward(cfg, weights, sequence, dtype=torch.float32)
+    del weights
+    agree, worst, worst_noise = 0, 0.0, 0.0
+    for i, tok in enumerate(tokens):
+        ref = logits[len(prompt) - 1 + i]
+        rms = float(ref.pow(2).mean().sqrt())
+        gap = float(ref.max() - ref[tok]) / rms           # how much the plain logits prefer another token
+        noise = float((rows[i] - ref).pow(2).mean().sqrt()) / rms
+        agree += int(ref.argmax()) == tok
+        worst, worst_noise = max(worst, gap), max(worst_noise, noise)
+    # bfloat16 rounds activations at a dozen places a layer: the logits carry noise of a few
+    # percent of their root mean square at this depth, and a token may win by less than that
+    noise_bound = 0.06 if dtype_name == "bf16" else 2e-4
+    record.update({"plain_agree": agree, "worst_gap_rms": round(worst, 5), "row_error_rms": round(worst_noise, 5),
+                   "bound_rms": noise_bound, "plain_seconds": round(time.perf_counter() - t0, 1)})
+    if worst_noise > noise_bound or worst > 6.5 * noise_bound:
+        raise RuntimeError(f"bench check: the engine's tokens are not the plain implementation's: {record}")
+    return record
 
 
 def weight_bytes_per_step(cfg, esize):
@@ -133,53 +211,71 @@ def main() -> int:
     pages_per_seq = -(-(PREFILL_TOKENS + NEW_TOKENS + prompt_len) // args.page_size)
     if args.long_prompt:
         max_seqs, pages_per_seq = 2, -(-(args.long_prompt + 16) // args.page_size)
-    engine = EngineCore(KVCoreConfig(
-        model_config=ModelConfig(model=".", dtype=args.dtype,
-                                 max_model_len=max(CONTEXT_LEN, args.long_prompt + 16)),
-        load_config=LoadConfig(load_format="random", seed=0),
-        cache_config=CacheConfig(block_size=args.page_size, num_gpu_blocks=max_seqs * pages_per_seq + 1),
-        scheduler_config=SchedulerConfig(max_num_seqs=max_seqs, max_num_scheduled_tokens=PREFILL_TOKENS,
-                                         max_num_partial_prefills=max_seqs,
-                                         max_long_partial_prefills=max_seqs),
-        device_config=DeviceConfig(device=device),
-    ), model=model)
+
+    def make_engine(max_model_len, seqs, pages):
+        return EngineCore(KVCoreConfig(
+            model_config=ModelConfig(model=".", dtype=args.dtype, max_model_len=max_model_len),
+            load_config=LoadConfig(load_format="random", seed=0),
+            cache_config=CacheConfig(block_size=args.page_size, num_gpu_blocks=pages),
+            scheduler_config=SchedulerConfig(max_num_seqs=seqs, max_num_scheduled_tokens=PREFILL_TOKENS,
+                                             max_num_partial_prefills=seqs, max_long_partial_prefills=seqs),
+            device_config=DeviceConfig(device=device),
+        ), model=model)
+
+    engine = make_engine(max(CONTEXT_LEN, args.long_prompt + 16), max_seqs, max_seqs * pages_per_seq + 1)
     rng = random.Random(0)
     vocab = cfg["vocab_size"]
     counter = [0]
+    check_mode = args.check or ("basic" if args.model == "70b" or args.only_prefill or args.mixed
+                                or args.long_prompt or args.sweep else "plain")
+    check = None
+    if check_mode != "none":
+        check = check_tokens(engine, cfg, check_mode, args.dtype)
+        print(f"[bench] check: {check}", file=sys.stderr, flush=True)
 
-    def new_request(n_prompt, n_new):
+    def new_request(n_prompt, n_new, eng=None):
         counter[0] += 1
         rid = f"bench-{counter[0]}"
         ids = [rng.randrange(vocab) for _ in range(n_prompt)]
-        engine.add_request(rid, SamplingParams(max_tokens=n_new, temperature=0.0, ignore_eos=True),
-                           prompt_token_ids=ids)
+        (eng or engine).add_request(rid, SamplingParams(max_tokens=n_new, temperature=0.0, ignore_eos=True),
+                                    prompt_token_ids=ids)
         return rid
 
     def drain():
         while engine.has_unfinished_requests():
             engine.step()
 
-    def decode_run(batch, steps, warmup):
+    def decode_run(batch, steps, warmup, eng=None, p_len=None):
         """tokens/s over exactly `steps` decode steps at `batch`, after `warmup` of them."""
-        slack = -(-batch * prompt_len // PREFILL_TOKENS) + 2  # steps others decode while prompts run
+        eng = eng or engine
+        p_len = p_len or prompt_len
+        slack = -(-batch * p_len // PREFILL_TOKENS) + 2  # steps others decode while prompts run
         for _ in range(batch):
-            new_request(prompt_len, warmup + steps + 1 + slack)
+            new_request(p_len, warmup + steps + 1 + slack, eng)
         # prompts first; a request samples its first token when its prompt ends
         while any(r.num_computed_tokens < r.num_prompt_tokens
-                  for r in engine.scheduler.requests.values()):
-            engine.step()
+                  for r in eng.scheduler.requests.values()):
+            eng.step()
         for _ in range(warmup):
-            engine.step()
-        ctx_start = prompt_len + 1 + warmup
+            eng.step()
+        ctx_start = p_len + 1 + warmup
         torch.cuda.synchronize()
         t_start = time.perf_counter()
         for _ in range(steps):
-            engine.step()
+            eng.step()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t_start
-        engine.abort_requests(None)
+        eng.abort_requests(None)
         mean_ctx = ctx_start + steps / 2
         return batch * steps / elapsed, elapsed / steps, mean_ctx
+
+    def decode_line(batch, steps, warmup, eng=None, p_len=None):
+        v, sec, ctx = decode_run(batch, steps, warmup, eng, p_len)
+        need = weight_bytes_per_step(cfg, esize) + kv_bytes(cfg, batch, ctx, esize)
+        return {"workload": "decode", "model": model_name, "dtype": args.dtype, "batch": batch,
+                "context": int(ctx), "tokens_per_s": round(v, 1), "ms_per_step": round(sec * 1e3, 4),
+                "gb_per_step": round(need / 1e9, 3), "hbm_gb_per_s": round(need / sec / 1e9, 1),
+                "hbm_frac": round(need / sec / HBM_PEAK, 4)}
 
     def prefill_run():
         times = []
@@ -193,6 +289,18 @@ def main() -> int:
             drain()
         return sorted(times[1:])[1]  # median of the three after the warm-up run
 
+    if args.sweep:
+        for b in (1, 2, 4, 8, 9, 12, 16, 24, 32, 48, 64):
+            print(json.dumps(decode_line(b, 48, 8)), flush=True)
+        del engine
+        for ctx_len, batches in ((8192, (1, 8)), (32768, (1, 8)), (131072, (1,))):
+            for b in batches:
+                room = ctx_len + 128
+                eng = make_engine(room, b, b * -(-room // args.page_size) + 1)
+                print(json.dumps(decode_line(b, 32, 4, eng, ctx_len - 48)), flush=True)
+                del eng
+                torch.cuda.empty_cache()
+        return 0
     if args.long_prompt:
         times = []
         for i in range(3):
@@ -260,6 +368,8 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)},
     }
+    if check is not None:
+        result["check"] = check
     if not args.no_points:
         sec = prefill_run()
         flops = prefill_flops(cfg, PREFILL_TOKENS)
@@ -267,10 +377,12 @@ def main() -> int:
                              "ms": round(sec * 1e3, 3),
                              "frac": round(flops / sec / PEAK_FLOPS[args.dtype], 4)}
         points = {}
-        for b in (1, 64):
+        for b in (1, 16, 32, 64):
             steps = max(16, min(args.steps, 64))
-            v, _, _ = decode_run(b, steps, min(args.warmup, 8))
+            v, sec_b, ctx_b = decode_run(b, steps, min(args.warmup, 8))
             points[f"decode_b{b}"] = round(v, 2)
+            need = weight_bytes_per_step(cfg, esize) + kv_bytes(cfg, b, ctx_b, esize)
+            points[f"decode_b{b}_hbm_frac"] = round(need / sec_b / HBM_PEAK, 4)
         result["points"] = points
     print(json.dumps(result), flush=True)
     return 0

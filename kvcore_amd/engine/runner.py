@@ -434,10 +434,13 @@ class ModelRunner:
         plan_len = min(plan_len, self.max_model_len)
         key = (bucket, plan_len)
 
-        def run() -> torch.Tensor:
+        def run(keep: list | None = None) -> torch.Tensor:
             ctx = self._context(bucket, bucket, [1] * bucket, [plan_len] * bucket, 1, plan_len)
             hidden = self.model.forward(ctx)
-            return self.model.compute_logits(ctx, hidden, self._dev["logit_rows"], bucket)
+            logits = self.model.compute_logits(ctx, hidden, self._dev["logit_rows"], bucket)
+            if keep is not None:  # nothing made in here dies before the capture has ended
+                keep.extend((ctx, hidden, logits))
+            return logits
 
         if key in self._graphs:
             graph, logits = self._graphs[key]
@@ -449,21 +452,31 @@ class ModelRunner:
             return run()[:num_live]
         graph = torch.cuda.CUDAGraph()
         self.buffers.frozen = True
-        # No garbage collection while the stream is capturing: a collection may free device
-        # or pinned memory or another graph that some dead object still holds, and the HIP
-        # runtime aborts the process when memory is freed during a capture.
+        # Nothing may be given back to the HIP runtime while the stream is capturing: freeing
+        # pinned memory, destroying another graph or releasing its memory pool then fails, and
+        # the failure ends the process.  Three guards.  (1) No garbage collection during the
+        # capture (and one before it): a collection may free an earlier runner with its pinned
+        # buffer and its graphs, held only by a reference cycle, at a time of its choosing.
+        # (2) The step buffers are frozen: a buffer that would have to grow (which drops the
+        # graphs) raises instead.  (3) What the captured step itself makes (its context, the
+        # views it returns) is kept in ``keep`` until the capture has ended, so no reference
+        # count reaches zero inside it.  Device memory that library calls take and give back
+        # inside the capture (the vendor product's workspace) belongs to the graph's pool,
+        # which the allocator does not return to the runtime while a capture runs.
         gc.collect()
         gc_was_enabled = gc.isenabled()
         gc.disable()
+        keep: list = []
         try:
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             with torch.cuda.graph(graph, pool=self._graph_pool):
-                logits = run()
+                logits = run(keep)
         finally:
             if gc_was_enabled:
                 gc.enable()
             self.buffers.frozen = False
+        del keep
         self._graphs[key] = (graph, logits)
         graph.replay()
         self.graph_replays += 1

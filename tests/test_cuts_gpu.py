@@ -573,3 +573,47 @@ def test_packed_weights_change_no_bit(models):
     for key, row in rows[True].items():
         assert torch.equal(row, rows[False][key]), key
     compare(rows[True], {"r": oracle("D", cfg, weights, tokens)}, torch.bfloat16)
+
+
+@pytest.mark.parametrize("name", ["A", "D"])
+def test_a_captured_step_allocates_and_frees_nothing_of_its_own(models, name, monkeypatch):
+    """While a decode step is captured into a graph, the step buffers are frozen and nothing
+    under the step may make or drop a tensor of its own (a free that reaches the HIP runtime
+    during a capture ends the process): torch's allocating constructors raise while the
+    buffers are frozen, every step buffer asked for must already be there, and torch's
+    allocator must hold after the capture what it held before it, apart from the graph's own
+    pool."""
+    from kvcore_amd.engine import context
+
+    folder, cfg, weights, page = models[name]
+    tokens = random_tokens(40, cfg["vocab_size"], seed=55)
+    session = session_for(folder, torch.bfloat16, page, max_tokens=64)
+    if not session.runner.use_hip_graphs:
+        pytest.skip("this model's steps are not captured")
+    frozen_gets = []
+    real_get = context.StepBuffers.get
+
+    def watched_get(self, name_, rows, cols, dtype, reserve=0):
+        if self.frozen:
+            buf = self._store.get(name_)
+            assert buf is not None and buf.dtype == dtype and buf.shape[1] == cols and buf.shape[0] >= rows, \
+                f"step buffer {name_!r} is not there at its full size during the capture"
+            frozen_gets.append(name_)
+        return real_get(self, name_, rows, cols, dtype, reserve)
+
+    monkeypatch.setattr(context.StepBuffers, "get", watched_get)
+    for fn in ("empty", "zeros", "ones", "full", "tensor", "empty_like", "zeros_like", "arange"):
+        real = getattr(torch, fn)
+
+        def guarded(*a, _real=real, _fn=fn, **kw):
+            assert not session.runner.buffers.frozen, f"torch.{_fn} was called while a step was captured"
+            return _real(*a, **kw)
+
+        monkeypatch.setattr(torch, fn, guarded)
+    steps = [{"step": 0, "entries": [{"id": "r", "tokens": tokens[:30], "want": [29]}], "end": []}]
+    steps += [{"step": j + 1, "entries": [{"id": "r", "tokens": [tokens[30 + j]], "want": [0]}], "end": []}
+              for j in range(6)]
+    got = collect(session, steps)
+    assert session.runner.graph_replays >= 4 and frozen_gets, "a step should have been captured"
+    assert not session.runner.buffers.frozen
+    compare(got, {"r": oracle(name, cfg, weights, tokens)}, torch.bfloat16)
