@@ -52,6 +52,9 @@ def parse_args(argv=None) -> argparse.Namespace:
                         "them (default: where the device has room)")
     p.add_argument("--num-gpu-blocks", type=int, default=None)
     p.add_argument("--gpu-memory-utilization", type=float, default=0.9)
+    p.add_argument("--poison-pages", action="store_true",
+                   help="debugging aid: fill every cache page with NaN when a request gets it and "
+                        "when it is given back")
     p.add_argument("--random-weights", action="store_true",
                    help="fill the parameters from --seed; the folder needs only config.json")
     p.add_argument("--seed", type=int, default=0)
@@ -113,7 +116,8 @@ def build_config(args: argparse.Namespace):
         load_config=LoadConfig(load_format="random" if args.random_weights else "safetensors",
                                seed=args.seed, pack_decode_weights=args.pack_decode_weights),
         cache_config=CacheConfig(block_size=args.block_size, num_gpu_blocks=args.num_gpu_blocks,
-                                 gpu_memory_utilization=args.gpu_memory_utilization),
+                                 gpu_memory_utilization=args.gpu_memory_utilization,
+                                 poison_pages=args.poison_pages),
         scheduler_config=SchedulerConfig(
             max_num_seqs=args.max_num_seqs,
             max_num_scheduled_tokens=args.max_num_scheduled_tokens,

@@ -241,6 +241,38 @@ class Block(Part):
         """Checkpoint sub-prefix -> part."""
         raise NotImplementedError
 
+    # ---- what any arrangement needs to let the products around a norm do the norm's work
+    # (see ``ops.ResidualSink``): which of the two ways a step of this size takes, and the
+    # sink itself.  A block that does not use them gets ordinary tensors and separate norms.
+    @staticmethod
+    def norm_folding(ctx: "StepContext", width: int) -> tuple[bool, bool]:
+        """``(fold, sums)`` for this step: ``fold``, very few rows of bfloat16: the product
+        before a norm adds into the residual and keeps sums of squares, the product after it
+        applies the scale factor (``ops.ScaledRows``); ``sums``, a few dozen rows: the product
+        before a norm leaves partial sums of slices along K and one kernel adds them into the
+        residual and normalises (``ops.NormedRows``).  Never both."""
+        from kvcore_amd.ops import library as ops
+
+        ok = width % 8 == 0
+        return (ok and ops.rows_fusable(ctx.num_tokens, ctx.dtype, width),
+                ok and ops.rows_sinkable(ctx.num_tokens, ctx.dtype, width))
+
+    @staticmethod
+    def residual_sink(ctx: "StepContext", residual: torch.Tensor, gain: "tuple[torch.Tensor, float]",
+                      name: str, fold: bool):
+        """The ``ops.ResidualSink`` that a part's last product goes into instead of a tensor:
+        ``gain`` is the following norm's ``as_gain()``, ``name`` the step buffer that receives
+        the rows for the part after the norm, ``fold`` as ``norm_folding`` says."""
+        from kvcore_amd.ops import library as ops
+
+        H = residual.shape[1]
+        rows = ctx.buf(name, H)
+        if fold:
+            parts = ctx.buffers.get(name + "_ss", ops.SKINNY_PREFERRED_ROWS, -(-H // 16), torch.float32)
+            return ops.ResidualSink(residual, gain[0], gain[1], rows, parts)
+        slices = ctx.buffers.get("block_slices", ops.mid_slices_bound(H) * ops.MID_ROWS, H, torch.float32)
+        return ops.ResidualSink(residual, gain[0], gain[1], rows, None, slices)
+
     def input_gain(self, scaled: bool = True) -> "tuple[torch.Tensor, float] | None":
         """``(gain, eps)`` of the block's first norm (see :meth:`Norm.as_gain`) if the block
         before may do that norm's work, else None: with ``scaled`` it hands over

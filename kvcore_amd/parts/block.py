@@ -46,25 +46,13 @@ class PreNormBlock(Block):
             return None
         return gain
 
-    @staticmethod
-    def _sink(ctx, residual: torch.Tensor, gain, name: str, fold: bool) -> ops.ResidualSink:
-        H = residual.shape[1]
-        rows = ctx.buf(name, H)
-        if fold:
-            parts = ctx.buffers.get(name + "_ss", ops.SKINNY_PREFERRED_ROWS, -(-H // 16), torch.float32)
-            return ops.ResidualSink(residual, gain[0], gain[1], rows, parts)
-        slices = ctx.buffers.get("block_slices", ops.mid_slices_bound(H) * ops.MID_ROWS, H, torch.float32)
-        return ops.ResidualSink(residual, gain[0], gain[1], rows, None, slices)
-
     def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
         # With very few rows of bfloat16 the norms fold into the products around them: the product
         # before a norm adds into the residual and keeps the sums of squares, the product after
         # it applies the scale factor.  Otherwise every norm is a kernel of its own.
         # With a few dozen rows the product before a norm leaves partial sums of slices along
         # K, and one kernel adds them into the residual and normalises.
-        H = residual.shape[1]
-        fold = ops.rows_fusable(ctx.num_tokens, ctx.dtype, H) and H % 8 == 0
-        sums = ops.rows_sinkable(ctx.num_tokens, ctx.dtype, H) and H % 8 == 0
+        fold, sums = self.norm_folding(ctx, residual.shape[1])
         if isinstance(delta, ops.ScaledRows):
             x = delta  # the block before made the first norm's rows
         elif isinstance(delta, ops.NormedRows):
@@ -78,7 +66,7 @@ class PreNormBlock(Block):
         if self.mixer.takes_sink and ((fold and self.ffn.takes_scaled_rows) or sums):
             gain = post.as_gain()
         if gain is not None:
-            x2 = self.mixer.forward(x, ctx, call, sink=self._sink(ctx, residual, gain, "block_x2", fold))
+            x2 = self.mixer.forward(x, ctx, call, sink=self.residual_sink(ctx, residual, gain, "block_x2", fold))
             if isinstance(x2, ops.NormedRows):
                 x2 = x2.data
         else:
@@ -90,7 +78,7 @@ class PreNormBlock(Block):
         if next_block is not None and self.ffn.takes_sink and (fold or sums):
             gain = next_block.input_gain(scaled=fold)
         if gain is not None:
-            return self.ffn.forward(x2, ctx, call, sink=self._sink(ctx, residual, gain, "block_x", fold))
+            return self.ffn.forward(x2, ctx, call, sink=self.residual_sink(ctx, residual, gain, "block_x", fold))
         return self.ffn.forward(x2, ctx, call)
 
 

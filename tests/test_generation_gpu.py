@@ -30,14 +30,14 @@ def folders(tmp_path_factory):
 
 
 def make_engine(folder, dtype, page, *, num_pages=None, max_seqs=4, budget=64, partial=4, threshold=0,
-                run_ahead=True, graphs=True):
+                run_ahead=True, graphs=True, poison=False):
     from kvcore_amd import (CacheConfig, DeviceConfig, KVCoreConfig, LoadConfig, ModelConfig, SchedulerConfig)
     from kvcore_amd.engine.llm_engine import LLMEngine
 
     return LLMEngine(KVCoreConfig(
         model_config=ModelConfig(model=str(folder), dtype=dtype),
         load_config=LoadConfig(seed=77),
-        cache_config=CacheConfig(block_size=page, num_gpu_blocks=num_pages),
+        cache_config=CacheConfig(block_size=page, num_gpu_blocks=num_pages, poison_pages=poison),
         scheduler_config=SchedulerConfig(max_num_seqs=max_seqs, max_num_scheduled_tokens=budget,
                                          max_num_partial_prefills=partial, max_long_partial_prefills=partial,
                                          long_prefill_token_threshold=threshold,
@@ -298,7 +298,8 @@ def test_preemption_with_seeded_sampling_and_steps_launched_ahead(folders, dtype
             for i, (rid, p) in enumerate(prompts.items())]
     results = {}
     for run_ahead in (False, True):
-        tight = make_engine(folder, dtype, page, num_pages=9, run_ahead=run_ahead)  # 8 usable pages
+        # 8 usable pages, each filled with NaN when it is taken and when it is given back
+        tight = make_engine(folder, dtype, page, num_pages=9, run_ahead=run_ahead, poison=True)
         results[run_ahead] = {o.request_id: o.output_token_ids for o in tight.generate(reqs)}
         assert tight.engine_core.scheduler.num_preemptions > 0
         assert tight.engine_core.kv_manager.num_free_pages() == [8]
