@@ -148,12 +148,16 @@ def check_tokens(engine, cfg, mode, dtype_name):
         noise = float((rows[i] - ref).pow(2).mean().sqrt()) / rms
         agree += int(ref.argmax()) == tok
         worst, worst_noise = max(worst, gap), max(worst_noise, noise)
-    # bfloat16 rounds activations at a dozen places a layer: the logits carry noise of a few
-    # percent of their root mean square at this depth, and a token may win by less than that
-    noise_bound = 0.06 if dtype_name == "bf16" else 2e-4
+    # bfloat16 rounds activations at a dozen places a layer, so a row of logits carries noise
+    # that grows like the square root of the depth: 0.9 to 1.2% of the row's root mean square
+    # at two layers of these sizes, 5.2% at 32.  The bound is 2% at two layers times
+    # sqrt(layers / 2); a wrong kernel, page or position gives 100% and more.  A token may
+    # lose to another by no more than a few times that noise.
+    layers = cfg["num_hidden_layers"]
+    noise_bound = round(0.02 * (layers / 2) ** 0.5, 4) if dtype_name == "bf16" else 2e-4
     record.update({"plain_agree": agree, "worst_gap_rms": round(worst, 5), "row_error_rms": round(worst_noise, 5),
                    "bound_rms": noise_bound, "plain_seconds": round(time.perf_counter() - t0, 1)})
-    if worst_noise > noise_bound or worst > 6.5 * noise_bound:
+    if worst_noise > noise_bound or worst > 5 * noise_bound:
         raise RuntimeError(f"bench check: the engine's tokens are not the plain implementation's: {record}")
     return record
 
