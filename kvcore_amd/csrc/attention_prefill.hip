@@ -285,62 +285,65 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
   for (int i = 0; i < V_PER_THREAD; ++i) {
     v_off[i] = (v_rem >> 1) * page_size + (v_rem & 1) * 8;
   }
-  // Element offsets of this wave's key blocks of the tile at kb0 in the K and V planes, or -1
-  // (no such block, or not a page).  They are looked up one tile before the tile is fetched (a
-  // lookup is a scalar load whose answer the fetch would otherwise wait for) and with as little
-  // scalar arithmetic as possible, which this kernel has much of: a shift where a page holds a
-  // power of two of key blocks, and one 64-bit product per block for both planes.
+  // Where the key blocks of a tile lie.  Lane i of every wave looks up key block kb0 + i of
+  // the tile with one vector load (`lookup_issue`), one tile before the tile is fetched; the
+  // page comes back while the tile before is worked on, and `lookup_finish` turns it into the
+  // element offsets of the block's K rows and V rows in their planes (-1: no such block, or
+  // not a page), which the fetch then reads as scalars from the lanes of its own key blocks.
+  // (Scalar loads, one per key block with a wait and three branches each, cost a tenth of the
+  // kernel.)
   const int sub_mask = blocks_per_page - 1;
   const int sub_shift = (blocks_per_page & sub_mask) == 0 ? __builtin_ctz(blocks_per_page) : -1;
   const int64_t page_elems = static_cast<int64_t>(nkv) * page_size * D;  // of one plane
   const int64_t head_elems = static_cast<int64_t>(hk) * page_size * D;
-  auto block_at = [&](int kb, int64_t& k_at, int64_t& v_at) {
-    k_at = v_at = -1;
-    if (kb < kb_end) {
-      int page_index, sub;
-      if (sub_shift >= 0) {
-        page_index = kb >> sub_shift;
-        sub = kb & sub_mask;
-      } else {
-        page_index = kb / blocks_per_page;
-        sub = kb - page_index * blocks_per_page;
-      }
-      const int page = __builtin_amdgcn_readfirstlane(row_table[page_index]);
-      if (page > 0 && page < num_pages) {
-        const int64_t at = page * page_elems + head_elems;
-        k_at = at + sub * (16 * D);
-        v_at = at + sub * 16;
-      }
+  const int lk_lane = lane & 15;
+  int lk_page = 0, lk_sub = 0;
+  auto lookup_issue = [&](int kb0) {
+    const int kb = kb0 + lk_lane;
+    const bool there = lk_lane < kKeyBlocks && kb < kb_end;
+    int page_index;
+    if (sub_shift >= 0) {  // uniform
+      page_index = kb >> sub_shift;
+      lk_sub = kb & sub_mask;
+    } else {
+      page_index = kb / blocks_per_page;
+      lk_sub = kb - page_index * blocks_per_page;
     }
+    lk_sub = there ? lk_sub : -1;
+    lk_page = row_table[there ? page_index : 0];
   };
   // whether step i of the K fetch and piece i of the V fetch lie in the same key block for all i
   constexpr bool kSameBlocks = ROWS_PER_STEP == 16 && V_GROUPS == 1;
-  auto lookup_pages = [&](int kb0, int64_t (&kbase)[K_PER_THREAD], int64_t (&vbase)[V_PER_THREAD]) {
-    if constexpr (kSameBlocks) {
-      static_assert(K_PER_THREAD == V_PER_THREAD, "one key block per step and piece");
+  auto lookup_finish = [&](int64_t (&kbase)[K_PER_THREAD], int64_t (&vbase)[V_PER_THREAD]) -> bool {
+    const bool ok = lk_sub >= 0 && lk_page > 0 && lk_page < num_pages;
+    const int64_t at = lk_page * page_elems + head_elems;
+    const int64_t k_at = ok ? at + lk_sub * (16 * D) : -1;
+    const int64_t v_at = ok ? at + lk_sub * 16 : -1;
+    auto pick = [&](int64_t v, int from) -> int64_t {
+      const uint32_t lo = __builtin_amdgcn_readlane(static_cast<int>(static_cast<uint64_t>(v) & 0xffffffffu), from);
+      const uint32_t hi = __builtin_amdgcn_readlane(static_cast<int>(static_cast<uint64_t>(v) >> 32), from);
+      return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+    };
 #pragma unroll
-      for (int i = 0; i < K_PER_THREAD; ++i) block_at(kb0 + i, kbase[i], vbase[i]);
-    } else {
-      int64_t unused;
+    for (int i = 0; i < K_PER_THREAD; ++i)
+      kbase[i] = pick(k_at, kSameBlocks ? i : (i * ROWS_PER_STEP) / 16 + k_block0);
 #pragma unroll
-      for (int i = 0; i < K_PER_THREAD; ++i)
-        block_at(kb0 + (i * ROWS_PER_STEP) / 16 + k_block0, kbase[i], unused);
-#pragma unroll
-      for (int i = 0; i < V_PER_THREAD; ++i) block_at(kb0 + v_group * V_PER_THREAD + i, unused, vbase[i]);
-    }
+    for (int i = 0; i < V_PER_THREAD; ++i) vbase[i] = pick(v_at, kSameBlocks ? i : v_group * V_PER_THREAD + i);
+    // every key block of the tile is there (lanes beyond the tile's blocks do not count)
+    return __ballot(ok || lk_lane >= kKeyBlocks) == ~0ull;
   };
-  auto fetch_tile = [&](int kb0, const int64_t (&kbase)[K_PER_THREAD], const int64_t (&vbase)[V_PER_THREAD]) {
+  auto fetch_tile = [&](int kb0, const int64_t (&kbase)[K_PER_THREAD], const int64_t (&vbase)[V_PER_THREAD],
+                        bool all_there) {
     const bool tail = (kb0 + kKeyBlocks) * 16 > pos_hi + 1;  // uniform: some keys are not the request's
-    if (!tail) {
-      // every key of the tile is the request's: a scalar base and a fixed offset per piece
+    if (!tail && all_there) {
+      // every key of the tile is the request's and on a page: a scalar base and a fixed offset
+      // per piece, and no branch between the loads
 #pragma unroll
       for (int i = 0; i < K_PER_THREAD; ++i)
-        kreg[i] = (kbase[i] >= 0) ? *reinterpret_cast<const uint4*>(k_cache + kbase[i] + k_off[i])
-                                  : make_uint4(0u, 0u, 0u, 0u);
+        kreg[i] = *reinterpret_cast<const uint4*>(k_cache + kbase[i] + k_off[i]);
 #pragma unroll
       for (int i = 0; i < V_PER_THREAD; ++i)
-        vreg[i] = (vbase[i] >= 0) ? *reinterpret_cast<const uint4*>(v_cache + vbase[i] + v_off[i])
-                                  : make_uint4(0u, 0u, 0u, 0u);
+        vreg[i] = *reinterpret_cast<const uint4*>(v_cache + vbase[i] + v_off[i]);
       return;
     }
 #pragma unroll
@@ -403,22 +406,40 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
   auto work_tile = [&](int kb0, int buf) {
     const bf16_t* k_lds = tiles + buf * TILE_ELEMS;
     const bf16_t* v_lds = k_lds + K_ELEMS;
-    // ---- raw scores of the tile for this wave's rows
+    // ---- raw scores of the tile for this wave's rows.  The operand reads of two key blocks
+    // are asked for while the matrix instructions of the two before them run (left to itself
+    // the compiler asks for each read one instruction before its use, and every matrix
+    // instruction then waits out the latency of LDS); the two blocks' sums are interleaved so
+    // that no instruction waits for the one before it.
     f32x4_t s[CT][kKeyBlocks];
+    constexpr int GK = (CT == 1) ? 2 : 1;  // key blocks a group
+    bf16x8_t ka[2][GK][NC];
+    auto read_keys = [&](int grp, bf16x8_t (&dst)[GK][NC]) {
 #pragma unroll
-    for (int kbi = 0; kbi < kKeyBlocks; ++kbi) {
-      bf16x8_t ka[NC];
-#pragma unroll
-      for (int c = 0; c < NC; ++c)
-        ka[c] = *reinterpret_cast<const bf16x8_t*>(k_lds + (kbi * 16 + col) * KROW + 32 * c + 8 * quad);
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) {
-        f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int b = 0; b < GK; ++b)
 #pragma unroll
         for (int c = 0; c < NC; ++c)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], qb[ct][c], acc, 0, 0, 0);
-        s[ct][kbi] = acc;
-      }
+          dst[b][c] = *reinterpret_cast<const bf16x8_t*>(k_lds + ((grp * GK + b) * 16 + col) * KROW + 32 * c + 8 * quad);
+    };
+    read_keys(0, ka[0]);
+#pragma unroll
+    for (int grp = 0; grp < kKeyBlocks / GK; ++grp) {
+      if (grp + 1 < kKeyBlocks / GK) read_keys(grp + 1, ka[(grp + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+      f32x4_t acc[CT][GK];
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+          for (int b = 0; b < GK; ++b)
+            acc[ct][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                ka[grp & 1][b][c], qb[ct][c], c == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : acc[ct][b], 0, 0, 0);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int b = 0; b < GK; ++b) s[ct][grp * GK + b] = acc[ct][b];
+      __builtin_amdgcn_sched_barrier(0);
     }
     // ---- softmax update per row over the 64 keys of the tile; a tile that every live row of
     // the wave sees whole needs no masks
@@ -482,17 +503,33 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
       ps += __shfl_xor(ps, 32, 64);
       l[ct] += ps;
     }
-    // ---- O^T += V^T P^T, two key blocks a product
+    // ---- O^T += V^T P^T, two key blocks a product; the operand reads run half a pair ahead
+    constexpr int GJ = NJ / (2 * CT);  // operand reads a group
+    constexpr int NG = NJ / GJ;        // groups a pair of key blocks
+    bf16x8_t va[2][GJ];
+    auto read_values = [&](int pr, int grp, bf16x8_t (&dst)[GJ]) {
+#pragma unroll
+      for (int jj = 0; jj < GJ; ++jj) {
+        const int j = grp * GJ + jj;
+        dst[jj] = *reinterpret_cast<const bf16x8_t*>(v_lds + (((pr * NJ + j) * 4 + quad) * 16 + (col ^ (8 * (quad >> 1)))) * 8);
+      }
+    };
+    read_values(0, 0, va[0]);
 #pragma unroll
     for (int pr = 0; pr < kKeyBlocks / 2; ++pr) {
       if ((kb0 + 2 * pr) * 16 > wave_pos_hi) break;  // scalar: later blocks weigh nothing
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        const bf16x8_t va =
-            *reinterpret_cast<const bf16x8_t*>(v_lds + (((pr * NJ + j) * 4 + quad) * 16 + (col ^ (8 * (quad >> 1)))) * 8);
+      for (int grp = 0; grp < NG; ++grp) {
+        const int step = pr * NG + grp;
+        if (grp + 1 < NG) read_values(pr, grp + 1, va[(step + 1) & 1]);
+        else if (pr + 1 < kKeyBlocks / 2) read_values(pr + 1, 0, va[(step + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-          o_acc[ct][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[ct][pr], o_acc[ct][j], 0, 0, 0);
+        for (int jj = 0; jj < GJ; ++jj)
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct)
+            o_acc[ct][grp * GJ + jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[step & 1][jj], pb[ct][pr], o_acc[ct][grp * GJ + jj], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
@@ -505,17 +542,19 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
   const int kb_mine_end = (kb_mine + tiles_mine * kKeyBlocks < kb_end) ? kb_mine + tiles_mine * kKeyBlocks : kb_end;
   if (kb_mine < kb_mine_end) {  // the same for the whole block
     int64_t kbase[K_PER_THREAD], vbase[V_PER_THREAD];
-    lookup_pages(kb_mine, kbase, vbase);
-    fetch_tile(kb_mine, kbase, vbase);
-    lookup_pages(kb_mine + kKeyBlocks, kbase, vbase);
+    lookup_issue(kb_mine);
+    bool all_there = lookup_finish(kbase, vbase);
+    fetch_tile(kb_mine, kbase, vbase, all_there);
+    lookup_issue(kb_mine + kKeyBlocks);
     store_tile(0);
     __syncthreads();
     int buf = 0;
     for (int kb0 = kb_mine; kb0 < kb_mine_end; kb0 += kKeyBlocks, buf ^= 1) {
       const bool more = kb0 + kKeyBlocks < kb_mine_end;
       if (more) {
-        fetch_tile(kb0 + kKeyBlocks, kbase, vbase);        // in flight while this tile is used
-        lookup_pages(kb0 + 2 * kKeyBlocks, kbase, vbase);  // answered by the time it is fetched
+        all_there = lookup_finish(kbase, vbase);
+        fetch_tile(kb0 + kKeyBlocks, kbase, vbase, all_there);  // in flight while this tile is used
+        lookup_issue(kb0 + 2 * kKeyBlocks);                     // answered by the time it is fetched
       }
       if (kb0 * 16 <= wave_pos_hi) work_tile(kb0, buf);  // scalar: else nothing here is visible to this wave
       if (more) store_tile(buf ^ 1);
