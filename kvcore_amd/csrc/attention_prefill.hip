@@ -48,6 +48,25 @@ __device__ __forceinline__ s16x4_t pack_bf16x4(const float* p) {
 }
 
 
+// A row of S^T lies in the four lanes col, col + 16, col + 32 and col + 48.  Their maximum and
+// their sum by the two lane-swap instructions of gfx950: registers only, where a shuffle goes
+// through LDS and back.
+typedef unsigned u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float quad_max(float v) {
+  const unsigned u = __float_as_uint(v);
+  const u32x2_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned w = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+  const u32x2_t b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_sum(float v) {
+  const unsigned u = __float_as_uint(v);
+  const u32x2_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned w = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+  const u32x2_t b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // KB: 16-key blocks per LDS tile
 template <int D, int KB>
 constexpr int tile_bytes() {
@@ -136,7 +155,7 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
   const int t_end = (t0 + bq < q_end) ? t0 + bq : q_end;
   const int n_tok = t_end - t0;
   const int pos_lo = positions[t0];
-  const int pos_hi = positions[t_end - 1];  // positions rise by one along a request's tokens
+  const int pos_hi = pos_lo + n_tok - 1;  // positions rise by one along a request's tokens
   const int first_lo = (window > 0 && pos_lo - window + 1 > 0) ? pos_lo - window + 1 : 0;
 
   // this lane's rows: column `col` of tile ct is row (wave*CT + ct)*16 + col of the block
@@ -150,7 +169,7 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
     live[ct] = tq < n_tok;
     my_tok[ct] = t0 + (live[ct] ? tq : 0);
     my_head[ct] = hk * g + rho % g;
-    my_pos[ct] = live[ct] ? positions[my_tok[ct]] : -1;
+    my_pos[ct] = live[ct] ? pos_lo + tq : -1;  // positions rise by one along a request's tokens
     my_first[ct] = (window > 0 && my_pos[ct] - window + 1 > 0) ? my_pos[ct] - window + 1 : 0;
     const bf16_t* qp = q + static_cast<int64_t>(my_tok[ct]) * q_stride +
                        static_cast<int64_t>(my_head[ct]) * D + 8 * quad;
@@ -213,30 +232,21 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
       }
     }
   }
-  // Bounds of what this wave's live rows can see.  They are the same in every lane after
-  // the exchange and are made scalar, so that the conditions on them below are scalar
-  // branches: matrix instructions must be skipped by a branch, never by a lane mask.
-  int wave_pos_hi = -1, wave_pos_lo = 0x7fffffff, wave_first_hi = 0;
-#pragma unroll
-  for (int ct = 0; ct < CT; ++ct) {
-    wave_pos_hi = max(wave_pos_hi, my_pos[ct]);
-    if (live[ct]) {
-      wave_pos_lo = min(wave_pos_lo, my_pos[ct]);
-      wave_first_hi = max(wave_first_hi, my_first[ct]);
-    }
-  }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    wave_pos_hi = max(wave_pos_hi, __shfl_xor(wave_pos_hi, o, 64));
-    wave_pos_lo = min(wave_pos_lo, __shfl_xor(wave_pos_lo, o, 64));
-    wave_first_hi = max(wave_first_hi, __shfl_xor(wave_first_hi, o, 64));
-  }
-  wave_pos_hi = __builtin_amdgcn_readfirstlane(wave_pos_hi);
-  wave_pos_lo = __builtin_amdgcn_readfirstlane(wave_pos_lo);
-  wave_first_hi = __builtin_amdgcn_readfirstlane(wave_first_hi);
+  // Bounds of what this wave's live rows can see, from the wave's first and last row alone
+  // (positions rise by one along the tokens).  They are scalars, so that the conditions on
+  // them below are scalar branches: matrix instructions must be skipped by a branch, never by
+  // a lane mask.
+  const int wave_tq_lo = (wave * CT * 16) / g;
+  const int wave_tq_hi = ((wave * CT + CT) * 16 - 1) / g;
+  const bool wave_live = wave_tq_lo < n_tok;
+  const int wave_pos_hi = wave_live ? pos_lo + (wave_tq_hi < n_tok ? wave_tq_hi : n_tok - 1) : -1;
+  const int wave_pos_lo = wave_live ? pos_lo + wave_tq_lo : 0x7fffffff;
+  const int wave_first_hi = (wave_live && window > 0 && wave_pos_hi - window + 1 > 0) ? wave_pos_hi - window + 1 : 0;
 
   f32x4_t o_acc[CT][NJ];
-  float m[CT], l[CT];  // m: the reference maximum of the raw (unscaled) scores
+  // m: the reference maximum of the raw (unscaled) scores, the same in the four lanes of a row;
+  // l: the sum of this lane's probabilities
+  float m[CT], l[CT];
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     m[ct] = -INFINITY;
@@ -441,6 +451,23 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
         for (int b = 0; b < GK; ++b) s[ct][grp * GK + b] = acc[ct][b];
       __builtin_amdgcn_sched_barrier(0);
     }
+    // with registers to spare the first value operands are asked for now: they do not depend
+    // on the softmax
+    constexpr bool kEarlyValues = CT == 1;
+    constexpr int GJ = NJ / (2 * CT);  // operand reads a group
+    constexpr int NG = NJ / GJ;        // groups a pair of key blocks
+    bf16x8_t va[2][GJ];
+    auto read_values = [&](int pr, int grp, bf16x8_t (&dst)[GJ]) {
+#pragma unroll
+      for (int jj = 0; jj < GJ; ++jj) {
+        const int j = grp * GJ + jj;
+        dst[jj] = *reinterpret_cast<const bf16x8_t*>(v_lds + (((pr * NJ + j) * 4 + quad) * 16 + (col ^ (8 * (quad >> 1)))) * 8);
+      }
+    };
+    if constexpr (kEarlyValues) {
+      read_values(0, 0, va[0]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     // ---- softmax update per row over the 64 keys of the tile; a tile that every live row of
     // the wave sees whole needs no masks
     const bool whole = (kb0 + kKeyBlocks) * 16 - 1 <= wave_pos_lo && kb0 * 16 >= wave_first_hi;
@@ -468,8 +495,7 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
       for (int kbi = 0; kbi < kKeyBlocks; ++kbi)
 #pragma unroll
         for (int i = 0; i < 4; ++i) v = fmaxf(v, s[ct][kbi][i]);
-      v = fmaxf(v, __shfl_xor(v, 16, 64));
-      v = fmaxf(v, __shfl_xor(v, 32, 64));
+      v = quad_max(v);
       mx[ct] = v;
       moved = moved || (v > m[ct] + unit);  // also true for the first visible key (m = -inf)
     }
@@ -499,22 +525,10 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
           pb[ct][kbi >> 1][4 * (kbi & 1) + i] = static_cast<__bf16>(p);
         }
       }
-      ps += __shfl_xor(ps, 16, 64);
-      ps += __shfl_xor(ps, 32, 64);
-      l[ct] += ps;
+      l[ct] += ps;  // this lane's keys only: the four lanes of a row are added up at the end
     }
     // ---- O^T += V^T P^T, two key blocks a product; the operand reads run half a pair ahead
-    constexpr int GJ = NJ / (2 * CT);  // operand reads a group
-    constexpr int NG = NJ / GJ;        // groups a pair of key blocks
-    bf16x8_t va[2][GJ];
-    auto read_values = [&](int pr, int grp, bf16x8_t (&dst)[GJ]) {
-#pragma unroll
-      for (int jj = 0; jj < GJ; ++jj) {
-        const int j = grp * GJ + jj;
-        dst[jj] = *reinterpret_cast<const bf16x8_t*>(v_lds + (((pr * NJ + j) * 4 + quad) * 16 + (col ^ (8 * (quad >> 1)))) * 8);
-      }
-    };
-    read_values(0, 0, va[0]);
+    if constexpr (!kEarlyValues) read_values(0, 0, va[0]);
 #pragma unroll
     for (int pr = 0; pr < kKeyBlocks / 2; ++pr) {
       if ((kb0 + 2 * pr) * 16 > wave_pos_hi) break;  // scalar: later blocks weigh nothing
@@ -564,6 +578,7 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
 
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
+    const float l_row = quad_sum(l[ct]);
     if (!live[ct]) continue;
     if (gridDim.z > 1) {
       // sums relative to m, and m in the exponent's units, as the combining kernel expects
@@ -574,11 +589,11 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
       for (int j = 0; j < NJ; ++j) *reinterpret_cast<f32x4_t*>(po + 16 * j) = o_acc[ct][j];
       if (quad == 0) {
         part_ml[2 * slot] = (m[ct] == -INFINITY) ? -INFINITY : m[ct] * scale_log2e;
-        part_ml[2 * slot + 1] = l[ct];
+        part_ml[2 * slot + 1] = l_row;
       }
       continue;
     }
-    const float inv = (l[ct] > 0.f) ? 1.f / l[ct] : 0.f;
+    const float inv = (l_row > 0.f) ? 1.f / l_row : 0.f;
     bf16_t* op = out + (static_cast<int64_t>(my_tok[ct]) * nh + my_head[ct]) * D + 4 * quad;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
