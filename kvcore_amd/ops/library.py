@@ -567,7 +567,7 @@ class ResidualSink:
     eps: float
     out: torch.Tensor
     ss_parts: torch.Tensor | None
-    # for steps of 9 to 64 rows: float32 room for the partial sums of a product cut along K
+    # for steps of 17 to 64 rows: float32 room for the partial sums of a product cut along K
     # (``mid_slices_bound(N) * T * N`` values); the sink then finishes the norm itself and
     # ``out`` receives the normalised rows
     slices: torch.Tensor | None = None
@@ -576,7 +576,7 @@ class ResidualSink:
 @dataclass
 class NormedRows:
     """Rows that a :class:`ResidualSink` has already added into the residual and normalised:
-    what ``linear`` returns for a sink that carries a workspace (steps of 9 to 64 rows)."""
+    what ``linear`` returns for a sink that carries a workspace (steps of 17 to 64 rows)."""
 
     data: torch.Tensor
 
@@ -584,22 +584,22 @@ class NormedRows:
 MID_ROWS = 64  # the most rows the weight-streaming kernels take
 
 
-FOLD_ROWS = 8  # up to here the few-row kernel with the norms folded in is the fastest (measured)
+# Up to here the few-row kernel with the norms folded in is the fastest.  Measured at 16 rows
+# against the kernels that share their rows through LDS: the 8B shape 4.13 against 4.45 ms a
+# step, the 70B shape 30.4 against 32.6, the 1B shape 1.13 against 1.11.
+FOLD_ROWS = 16
 
 
-def rows_fusable(num_rows: int, dtype: torch.dtype, width: int = 0) -> bool:
-    """Whether a step of ``num_rows`` tokens hands its norms to the products around them:
-    up to 8 rows, and up to 16 where the model's ``width`` is no multiple of 512, which the
-    kernel for more rows wants."""
-    most = FOLD_ROWS if width % 512 == 0 and width > 0 else SKINNY_PREFERRED_ROWS
-    return dtype == torch.bfloat16 and 0 < num_rows <= most
+def rows_fusable(num_rows: int, dtype: torch.dtype) -> bool:
+    """Whether a step of ``num_rows`` tokens hands its norms to the products around them: up
+    to 16 rows of bfloat16."""
+    return dtype == torch.bfloat16 and 0 < num_rows <= FOLD_ROWS
 
 
-def rows_sinkable(num_rows: int, dtype: torch.dtype, width: int = 0) -> bool:
+def rows_sinkable(num_rows: int, dtype: torch.dtype) -> bool:
     """Whether a step of ``num_rows`` tokens sends the products before its norms into a
-    :class:`ResidualSink` that finishes the norm itself: more rows than ``rows_fusable``
-    allows, at most 64."""
-    return dtype == torch.bfloat16 and not rows_fusable(num_rows, dtype, width) and 0 < num_rows <= MID_ROWS
+    :class:`ResidualSink` that finishes the norm itself: 17 to 64 rows."""
+    return dtype == torch.bfloat16 and FOLD_ROWS < num_rows <= MID_ROWS
 
 
 def skinny_blocks(N: int, K: int, gated: bool = False, packed: bool = False) -> int:
@@ -729,7 +729,7 @@ def add_slices_rmsnorm(out: torch.Tensor, residual: torch.Tensor, partial: torch
 
 
 def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None) -> NormedRows:
-    """A product of 9 to 64 rows into a sink: partial sums of slices along K, then one kernel
+    """A product of 17 to 64 rows into a sink: partial sums of slices along K, then one kernel
     that adds them into the residual and normalises.  Shapes the weight-streaming kernel does
     not take run the vendor product into the same workspace first."""
     M, K = x.shape
@@ -773,7 +773,7 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
         raise KernelError("linear_silu_mul: shapes do not match")
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and x.is_cuda and _skinny_operands_ok(x, w)
-            and (M <= FOLD_ROWS or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and not mid_operands_ok(x, w)))):
+            and M <= FOLD_ROWS):
         if M == 0:
             return
         if bias is not None and (bias.dtype != torch.bfloat16 or bias.shape != (2 * I,)):
@@ -786,7 +786,7 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and x.is_cuda and FOLD_ROWS < M <= MID_ROWS and mid_operands_ok(x, w)
             and out.stride(1) == 1):
-        # 9 to 64 rows: the waves of a block share the rows through LDS
+        # 17 to 64 rows: the waves of a block share the rows through LDS
         gemm_mid(out, x, w, bias, mode=1)
         return
     gate_up = scratch()
@@ -801,7 +801,7 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
     vendor matrix product through torch.  All sum in float32, and a float32 ``out`` receives
     the sums unrounded on either path.  With a :class:`ScaledRows` for ``x`` or a :class:`ResidualSink` for ``out``
     (few rows of bfloat16 only) the norm before or after the product is folded into it; a
-    sink returns the :class:`ScaledRows` it made, or, in a step of 9 to 64 rows, where it
+    sink returns the :class:`ScaledRows` it made, or, in a step of 17 to 64 rows, where it
     finishes the norm itself, :class:`NormedRows`."""
     if isinstance(out, ResidualSink) and out.slices is not None:
         if isinstance(x, ScaledRows):

@@ -246,7 +246,7 @@ class Block(Part):
     # sink itself.  A block that does not use them gets ordinary tensors and separate norms.
     @staticmethod
     def norm_folding(ctx: "StepContext", width: int) -> tuple[bool, bool]:
-        """``(fold, sums)`` for this step: ``fold``, very few rows of bfloat16: the product
+        """``(fold, sums)`` for this step: ``fold``, up to 16 rows of bfloat16: the product
         before a norm adds into the residual and keeps sums of squares, the product after it
         applies the scale factor (``ops.ScaledRows``); ``sums``, a few dozen rows: the product
         before a norm leaves partial sums of slices along K and one kernel adds them into the
@@ -254,8 +254,8 @@ class Block(Part):
         from kvcore_amd.ops import library as ops
 
         ok = width % 8 == 0
-        return (ok and ops.rows_fusable(ctx.num_tokens, ctx.dtype, width),
-                ok and ops.rows_sinkable(ctx.num_tokens, ctx.dtype, width))
+        return (ok and ops.rows_fusable(ctx.num_tokens, ctx.dtype),
+                ok and ops.rows_sinkable(ctx.num_tokens, ctx.dtype))
 
     @staticmethod
     def residual_sink(ctx: "StepContext", residual: torch.Tensor, gain: "tuple[torch.Tensor, float]",

@@ -45,18 +45,14 @@ def test_row_counts_choose_how_norms_and_products_meet():
     from kvcore_amd.ops import library as ops
 
     bf16, f32 = torch.bfloat16, torch.float32
-    # a width the kernels for a few dozen rows take: the fold stops at 8 rows
-    assert ops.rows_fusable(1, bf16, 4096) and ops.rows_fusable(8, bf16, 4096)
-    assert not ops.rows_fusable(9, bf16, 4096) and ops.rows_sinkable(9, bf16, 4096)
-    assert ops.rows_sinkable(64, bf16, 4096) and not ops.rows_sinkable(65, bf16, 4096)
-    # a narrow model keeps the fold up to 16 rows
-    assert ops.rows_fusable(16, bf16, 128) and not ops.rows_sinkable(16, bf16, 128)
-    assert ops.rows_sinkable(17, bf16, 128)
+    # the products do the norms' work up to 16 rows; from 17 to 64 a kernel of its own finishes them
+    assert ops.rows_fusable(1, bf16) and ops.rows_fusable(16, bf16)
+    assert not ops.rows_fusable(17, bf16) and ops.rows_sinkable(17, bf16)
+    assert ops.rows_sinkable(64, bf16) and not ops.rows_sinkable(65, bf16)
     # never both, and float32 neither
     for rows in range(0, 80):
-        for width in (96, 512, 4096):
-            assert not (ops.rows_fusable(rows, bf16, width) and ops.rows_sinkable(rows, bf16, width))
-            assert not ops.rows_fusable(rows, f32, width) and not ops.rows_sinkable(rows, f32, width)
+        assert not (ops.rows_fusable(rows, bf16) and ops.rows_sinkable(rows, bf16))
+        assert not ops.rows_fusable(rows, f32) and not ops.rows_sinkable(rows, f32)
 
 
 def test_slices_along_k_stay_within_the_bound_a_block_reserves_for():

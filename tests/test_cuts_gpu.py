@@ -417,8 +417,8 @@ def test_steps_of_a_few_dozen_rows_on_a_wide_model(tmp_path, monkeypatch):
 
     monkeypatch.setattr(ops, "gemm_mid", spy)
     n_req = 40
-    tail = 3  # tokens that the first twelve requests decode after the others have ended
-    seqs = {f"m{i}": random_tokens(5 + i % 7 + 10 + (tail if i < 12 else 0), cfg["vocab_size"], seed=800 + i)
+    tail = 3  # tokens that the first twenty requests decode after the others have ended
+    seqs = {f"m{i}": random_tokens(5 + i % 7 + 10 + (tail if i < 20 else 0), cfg["vocab_size"], seed=800 + i)
             for i in range(n_req)}
     seqs["late"] = random_tokens(50, cfg["vocab_size"], seed=899)
     total = sum(-(-len(t) // 64) * 64 for t in seqs.values())
@@ -426,7 +426,7 @@ def test_steps_of_a_few_dozen_rows_on_a_wide_model(tmp_path, monkeypatch):
     expect = {rid: plain.llama_forward(cfg, weights, t, dtype=torch.float64) for rid, t in seqs.items()}
     ids = [r for r in seqs if r != "late"]
     steps, k = [], 0
-    first = {r: len(seqs[r]) - 10 - (tail if i < 12 else 0) for i, r in enumerate(ids)}
+    first = {r: len(seqs[r]) - 10 - (tail if i < 20 else 0) for i, r in enumerate(ids)}
     for i in range(0, n_req, 8):
         steps.append({"step": k, "end": [], "entries": [
             {"id": r, "tokens": seqs[r][:first[r]], "want": [first[r] - 1]} for r in ids[i:i + 8]]})
@@ -441,11 +441,11 @@ def test_steps_of_a_few_dozen_rows_on_a_wide_model(tmp_path, monkeypatch):
             n = (9, 2, 13)[(3, 4, 7).index(j)]
             entries.append({"id": "late", "tokens": seqs["late"][late_at:late_at + n], "want": list(range(n))})
             late_at += n
-        steps.append({"step": k, "end": ids[12:] if j == 9 else [], "entries": entries}); k += 1
-    for j in range(tail):  # twelve rows: the same kernels from nine rows on
+        steps.append({"step": k, "end": ids[20:] if j == 9 else [], "entries": entries}); k += 1
+    for j in range(tail):  # twenty rows: the same kernels from seventeen rows on
         steps.append({"step": k, "end": [], "entries": [
-            {"id": r, "tokens": [seqs[r][fed[r]]], "want": [0]} for r in ids[:12]]}); k += 1
-        for r in ids[:12]:
+            {"id": r, "tokens": [seqs[r][fed[r]]], "want": [0]} for r in ids[:20]]}); k += 1
+        for r in ids[:20]:
             fed[r] += 1
     got = collect(session, steps)
     assert all(fed[r] == len(seqs[r]) for r in ids)
@@ -464,7 +464,7 @@ def test_layer_sizes_of_the_8b_model(tmp_path):
     """One layer with the widths of Llama-3-8B (4096 wide, 32 heads of 128 over 8 kv heads,
     14336 in the feed-forward) and a small vocabulary, against the plain implementation in
     float32: the shapes that decide which kernel runs are the real ones.  Prompts whole, then
-    12 rows together (the kernels that share the rows through LDS), then 3 (the few-row
+    20 rows together (the kernels that share the rows through LDS), then 12 and 3 (the few-row
     kernels with the norms folded in), through graphs where the runner uses them."""
     config = {
         "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 1,
@@ -477,10 +477,10 @@ def test_layer_sizes_of_the_8b_model(tmp_path):
     }
     folder = make_model_dir(tmp_path / "wide8b", config, seed=5)
     cfg, weights = plain.load_model_folder(folder)
-    n_req, tail = 12, 6
+    n_req, tail = 20, 6
     seqs = {f"r{i}": random_tokens(20 + 3 * i + tail, cfg["vocab_size"], seed=900 + i) for i in range(n_req)}
     total = sum(-(-len(t) // 64) * 64 for t in seqs.values())
-    session = session_for(folder, torch.bfloat16, 16, max_tokens=total, max_num_seqs=16)
+    session = session_for(folder, torch.bfloat16, 16, max_tokens=total, max_num_seqs=24)
     expect = {rid: plain.llama_forward(cfg, weights, t, dtype=torch.float32).double() for rid, t in seqs.items()}
     ids = list(seqs)
     steps, k = [], 0
@@ -491,8 +491,9 @@ def test_layer_sizes_of_the_8b_model(tmp_path):
         k += 1
     fed = {r: len(seqs[r]) - tail for r in ids}
     for j in range(tail):
-        live = ids if j < 3 else ids[:3]
-        steps.append({"step": k, "end": ids[3:] if j == 2 else [], "entries": [
+        live = ids if j < 2 else (ids[:12] if j < 4 else ids[:3])
+        ended = ids[12:] if j == 1 else (ids[3:12] if j == 3 else [])
+        steps.append({"step": k, "end": ended, "entries": [
             {"id": r, "tokens": [seqs[r][fed[r]]], "want": [0]} for r in live]})
         k += 1
         for r in live:
