@@ -196,7 +196,13 @@ def main(argv=None) -> int:
         engine = LLMEngine(config)
         engine_elapsed = time.perf_counter() - engine_start
         print(f"engine_init_sec={engine_elapsed:.3f}")
-        print(f"num_gpu_blocks={engine.engine_core.num_pages}")
+        core = engine.engine_core
+        print(f"num_gpu_blocks={core.num_pages}")
+        print(f"kv_bytes_per_block={core.bytes_per_page()}")
+        print(f"kv_cache_bytes={core.runner.cache_bytes()}")
+        if core.memory_profile is not None:  # the cache was sized by the profile steps
+            for name, value in vars(core.memory_profile).items():
+                print(f"memory_profile.{name}={value}")
 
         requests = build_generation_requests(args, engine.engine_core.model.spec.vocab_size)
         print("\n=== Requests ===")
@@ -224,6 +230,15 @@ def main(argv=None) -> int:
         print(f"engine_init_sec={engine_elapsed:.3f}")
         print(f"generate_sec={generate_elapsed:.3f}")
         print(f"total_elapsed_sec={time.perf_counter() - program_start:.3f}")
+        if args.device.startswith("cuda"):
+            import torch
+
+            free, total = torch.cuda.mem_get_info(torch.device(args.device))
+            print("\n=== Device Memory ===")
+            print(f"device_total_bytes={total}")
+            print(f"device_used_bytes={total - free}")
+            print(f"torch_reserved_bytes={torch.cuda.memory_reserved(torch.device(args.device))}")
+            print(f"torch_peak_allocated_bytes={torch.cuda.max_memory_allocated(torch.device(args.device))}")
     return 0
 
 

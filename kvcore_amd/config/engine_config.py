@@ -101,18 +101,23 @@ class CacheConfig:
 
 @dataclass(frozen=True)
 class SchedulerConfig:
-    """Reference: config.py:63-93 (same five names, same validation).  ``decode_run_ahead``
+    """Reference: config.py:63-93 (same five names, same validation).
+    ``max_num_partial_prefills`` left unset means ``max_num_seqs``: every request that fits
+    may be in its prompt at once (the reference's own default is 1, and its command line
+    raises it to 128: scripts/run_llm_engine_offline_batch.py:145).  ``decode_run_ahead``
     is this engine's own: while requests only decode, the next step is launched before the
     tokens of the step in flight have reached the host (``Scheduler.plan_decode_ahead``)."""
 
     max_num_seqs: int = 8
     max_num_scheduled_tokens: int = 512
-    max_num_partial_prefills: int = 1
+    max_num_partial_prefills: int | None = None
     max_long_partial_prefills: int = 1
     long_prefill_token_threshold: int = 0
     decode_run_ahead: bool = True
 
     def __post_init__(self) -> None:
+        if self.max_num_partial_prefills is None:
+            object.__setattr__(self, "max_num_partial_prefills", self.max_num_seqs)
         for name in (
             "max_num_seqs", "max_num_scheduled_tokens",
             "max_num_partial_prefills", "max_long_partial_prefills",

@@ -32,25 +32,32 @@ class LayerCall:
 
 @dataclass
 class CacheGroupView:
-    """Device side of one cache group: ``kv`` is the storage ``[planes, 2, pages, kv_heads,
-    page_size, head_dim]`` (index 0 keys, 1 values; see ``planes`` for the values' layout); ``table`` is ``[max_seqs, max_pages_per_seq]`` int32, row =
-    request slot, entry = page id (0 is the null page)."""
+    """Device side of one cache group.  ``storage[p]`` holds plane ``p`` of the group's need
+    for every schedule entry of the group: ``[entries, pages, page_size * elements a token]``,
+    a page being one contiguous row.  ``table`` is ``[max_seqs, max_pages_per_seq]`` int32,
+    row = request slot, entry = page id (0 is the null page)."""
 
-    kv: torch.Tensor
+    storage: list[torch.Tensor]
     table: torch.Tensor
     page_size: int
     window: int = 0
 
-    def planes(self, cache_index: int) -> tuple[torch.Tensor, torch.Tensor]:
-        """K plane ``[pages, kv_heads, page_size, head_dim]`` and V plane ``[pages, kv_heads,
-        head_dim, page_size]`` (a V page keeps its keys contiguous) of one cache index."""
+    @property
+    def num_pages(self) -> int:
+        return self.storage[0].shape[1]
+
+    def plane(self, cache_index: int, plane: int, *page_shape: int) -> torch.Tensor:
+        """The pages of one plane of one schedule entry: ``[pages, *page_shape]`` (a view;
+        ``page_shape`` must hold ``page_size`` tokens' worth of the plane, and defaults to one
+        flat row a page).  Attention views its keys as ``(kv_heads, page_size, head_dim)`` and
+        its values as ``(kv_heads, head_dim, page_size)``: a V page keeps the keys contiguous."""
         views = self.__dict__.setdefault("_plane_views", {})
-        got = views.get(cache_index)
+        key = (cache_index, plane, page_shape)
+        got = views.get(key)
         if got is None:
-            k = self.kv[cache_index, 0]
-            pages, heads, page_size, d = k.shape
-            got = (k, self.kv[cache_index, 1].view(pages, heads, d, page_size))
-            views[cache_index] = got
+            flat = self.storage[plane][cache_index]
+            got = flat.view(flat.shape[0], *page_shape) if page_shape else flat
+            views[key] = got
         return got
 
 

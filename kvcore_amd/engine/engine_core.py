@@ -42,6 +42,23 @@ class FinishedRequestOutput:
     finish_reason: FinishReason | None
 
 
+@dataclass(frozen=True)
+class MemoryProfile:
+    """What the profile steps measured, in bytes, and the page count that follows."""
+
+    total: int
+    free: int
+    others: int  # held on the device by anything but torch's allocator
+    live: int  # tensors that stay: weights, step buffers, workspaces, the graphs' pool
+    transient: int  # what a step takes and gives back
+    margin: int
+    budget: int
+    bytes_per_page: int
+    pages: int
+    useful_pages: int
+    formula_pages: int
+
+
 @dataclass
 class StepStats:
     """Wall-clock seconds of the last step's parts (the reference keeps the same in
@@ -89,23 +106,34 @@ class EngineCore:
         cache = config.cache_config
         self.max_model_len = config.model_config.max_model_len or model.spec.max_position_embeddings
         self.page_size = cache.block_size
+        self.sampler = Sampler(device, sched.max_num_seqs, engine_seed=config.load_config.seed)
         # ``num_pages`` counts pages of ``block_size`` tokens (with the null page); a cache
-        # group whose mixers want another page size holds the same number of tokens
-        self.num_pages = self._decide_num_pages()
-        self.group_configs = plan_groups([g.need for g in model.cache_groups], self.page_size, self.num_pages)
-        self.kv_manager = KVManager(self.group_configs, max_num_seqs=sched.max_num_seqs,
-                                    max_model_len=self.max_model_len, track_freed=cache.poison_pages)
-        self.scheduler = Scheduler(sched, self.kv_manager, max_model_len=self.max_model_len)
-        self.runner = ModelRunner(model, page_size=[g.page_size for g in self.group_configs],
-                                  num_pages=[g.num_pages for g in self.group_configs],
+        # group whose mixers want another page size holds the same number of tokens.  With no
+        # count given, the runner is built on a cache just large enough for the profile steps,
+        # which tell how much room is left, and the cache is then allocated anew
+        self.memory_profile: MemoryProfile | None = None
+        profiled = (cache.num_gpu_blocks is None and cache.profile_kv_cache and model.device.type == "cuda"
+                    and bool(model.cache_groups))
+        first_pages = self._profile_pages() if profiled else self._pages_without_profile()
+        first_groups = plan_groups([g.need for g in model.cache_groups], self.page_size, first_pages)
+        self.runner = ModelRunner(model, page_size=[g.page_size for g in first_groups],
+                                  num_pages=[g.num_pages for g in first_groups],
                                   max_num_seqs=sched.max_num_seqs,
                                   max_num_tokens=sched.max_num_scheduled_tokens,
                                   max_model_len=self.max_model_len,
                                   use_hip_graphs=config.device_config.use_hip_graphs,
                                   poison_pages=cache.poison_pages)
+        self.num_pages = first_pages
+        self.group_configs = first_groups
+        if profiled:
+            self.num_pages = self._measure_num_pages(first_pages)
+            self.group_configs = plan_groups([g.need for g in model.cache_groups], self.page_size, self.num_pages)
+            self.runner.resize_cache([g.num_pages for g in self.group_configs])
+        self.kv_manager = KVManager(self.group_configs, max_num_seqs=sched.max_num_seqs,
+                                    max_model_len=self.max_model_len, track_freed=cache.poison_pages)
+        self.scheduler = Scheduler(sched, self.kv_manager, max_model_len=self.max_model_len)
         if cache.poison_pages:
             self.runner.fill_cache(float("nan"))
-        self.sampler = Sampler(device, sched.max_num_seqs, engine_seed=config.load_config.seed)
         self.tokenizer_manager = None
         if model_json:
             self.tokenizer_manager = TokenizerManager.from_model_source(
@@ -125,26 +153,111 @@ class EngineCore:
 
     # ---------------------------------------------------------------------- capacity
     def bytes_per_page(self) -> int:
-        """Bytes that ``block_size`` tokens take in the cache, over all groups and planes."""
-        return sum(g.num_planes * 2 * g.need.num_kv_heads * self.page_size * g.need.head_dim
+        """Bytes that ``block_size`` tokens take in the cache, over all groups, entries and
+        planes (what a group keeps per token is its need's ``planes``)."""
+        return sum(g.num_planes * sum(g.need.token_elems()) * self.page_size
                    * torch.empty((), dtype=g.need.dtype or self.dtype).element_size()
                    for g in self.model.cache_groups)
 
-    def _decide_num_pages(self) -> int:
-        """An explicit ``num_gpu_blocks`` wins.  Otherwise: free device memory times the
-        utilisation, minus an estimate of the step buffers and a fixed margin, divided by
-        the bytes of one page over all planes; never more than every slot at full length
-        needs (reference: model_runner.py:696-768 measures the activation peak with a
-        dummy forward; the buffers here have known sizes)."""
+    def useful_pages(self) -> int:
+        """More pages than this no traffic can hold: every slot at the longest length."""
+        return self.config.scheduler_config.max_num_seqs * cdiv(self.max_model_len, self.page_size) + 1
+
+    def _pages_without_profile(self) -> int:
+        cache = self.config.cache_config
+        return cache.num_gpu_blocks if cache.num_gpu_blocks is not None else self.useful_pages()
+
+    def _profile_pages(self) -> int:
+        """Pages of the cache that the profile steps run on: room for one step's tokens."""
+        sched = self.config.scheduler_config
+        return min(self.useful_pages(), cdiv(sched.max_num_scheduled_tokens, self.page_size) + 2)
+
+    def _run_profile_steps(self) -> None:
+        """The largest step of each kind on the engine's own runner and sampler, so that every
+        step buffer, workspace and graph pool is there at its largest: a step of
+        ``max_num_scheduled_tokens`` prompt tokens (in as few requests as ``max_model_len``
+        allows), sampled both ways, then a step of single tokens for every slot, three times
+        (launch by launch, captured, replayed).  Pages are dealt round and round from the small
+        cache: what the steps compute is thrown away."""
+        sched = self.config.scheduler_config
+        runner = self.runner
+        counters = [0] * len(runner.groups)
+
+        def pages_for(tokens: int) -> list[list[int]]:
+            out = []
+            for g, grp in enumerate(runner.groups):
+                ids = []
+                for _ in range(cdiv(tokens, grp.page_size)):
+                    ids.append(1 + counters[g] % (grp.num_pages - 1))
+                    counters[g] += 1
+                out.append(ids)
+            return out
+
+        def sample_both_ways(logits: torch.Tensor) -> None:
+            n = logits.shape[0]
+            greedy = SamplingParams(max_tokens=1, temperature=0.0)
+            drawn = SamplingParams(max_tokens=1, temperature=1.0, top_k=50, top_p=0.9)
+            self.sampler.launch(logits, [SamplingRow(greedy, 0, 0)] * n).result()
+            self.sampler.launch(logits, [SamplingRow(drawn, i, 0) for i in range(n)]).result()
+
+        left = sched.max_num_scheduled_tokens
+        entries = []
+        while left > 0 and len(entries) < sched.max_num_seqs:
+            n = min(left, self.max_model_len)
+            slot = len(entries)
+            entries.append(StepEntry(f"profile-p{slot}", slot, 0, [0] * n, pages_for(n), (n - 1,)))
+            left -= n
+        sample_both_ways(runner.step(entries).logits)
+        singles = min(sched.max_num_seqs, sched.max_num_scheduled_tokens)
+        entries = [StepEntry(f"profile-d{slot}", slot, 0, [0], pages_for(1), (0,)) for slot in range(singles)]
+        for _ in range(3):
+            sample_both_ways(runner.step(entries).logits)
+
+    def _measure_num_pages(self, profile_pages: int) -> int:
+        """How many pages fit, by measurement (reference: model_runner.py:696-768 runs a dummy
+        forward at ``max_num_scheduled_tokens``, reads torch's peak and gives the cache what
+        ``gpu_memory_utilization`` of the device leaves beside it).  Here the profile steps run
+        on the engine's own runner, so what they allocate stays and is counted as it is:
+        ``live`` (weights, step buffers, workspaces, the graphs' pool), plus ``transient``, what
+        a step takes and gives back, plus what others hold on the device.  Never more than
+        every slot at full length needs.  The estimate by formula that stood here before is
+        logged beside the measurement."""
+        cache = self.config.cache_config
+        device = self.model.device
+        per_page = max(self.bytes_per_page(), 1)
+        torch.cuda.synchronize(device)
+        torch.cuda.reset_peak_memory_stats(device)
+        self._run_profile_steps()
+        torch.cuda.synchronize(device)
+        peak = torch.cuda.max_memory_allocated(device)
+        now = torch.cuda.memory_allocated(device)
+        live = now - self.runner.cache_bytes()
+        transient = max(peak - now, 0)
+        free, total = torch.cuda.mem_get_info(device)
+        others = max((total - free) - torch.cuda.memory_reserved(device), 0)
+        margin = 512 << 20  # for graphs of further batch sizes and what the allocator cannot pack
+        budget = int(total * cache.gpu_memory_utilization) - others - live - transient - margin
+        pages = int(budget // per_page)
+        useful = self.useful_pages()
+        formula = self._estimate_num_pages_by_formula(free + self.runner.cache_bytes(), total)
+        self.memory_profile = MemoryProfile(total, free, others, live, transient, margin, budget, per_page,
+                                            min(pages, useful), useful, formula)
+        logger.info("KV cache by measurement: total %.2f GiB, others %.2f, live %.2f, transient %.2f, "
+                    "margin %.2f, budget %.2f GiB, %d bytes a page -> %d pages (useful %d; the formula "
+                    "says %d, off by %+.1f%%)", total / 2**30, others / 2**30, live / 2**30,
+                    transient / 2**30, margin / 2**30, budget / 2**30, per_page, pages, useful, formula,
+                    100.0 * (formula - pages) / max(pages, 1))
+        if pages < 2:
+            raise RuntimeError(
+                f"not enough device memory for a KV cache: {total / 2**30:.1f} GiB in all, "
+                f"{(others + live + transient) / 2**30:.2f} GiB taken by weights, step buffers and "
+                f"others, {per_page} bytes per page")
+        return min(pages, useful)
+
+    def _estimate_num_pages_by_formula(self, free: int, total: int) -> int:
+        """The cross-check: step buffers guessed from the model's widths."""
         cache = self.config.cache_config
         sched = self.config.scheduler_config
-        if cache.num_gpu_blocks is not None:
-            return cache.num_gpu_blocks
-        per_page = max(self.bytes_per_page(), 1)
-        useful = sched.max_num_seqs * cdiv(self.max_model_len, self.page_size) + 1
-        if not cache.profile_kv_cache or self.model.device.type != "cuda":
-            return useful
-        free, total = torch.cuda.mem_get_info(self.model.device)
         esize = torch.empty((), dtype=self.dtype).element_size()
         spec = self.model.spec
         widest = max((p.shape[0] for bp in self.model.params.values() for p in [bp.spec]
@@ -152,14 +265,8 @@ class EngineCore:
         per_token = 4 * spec.hidden_size + esize * (4 * spec.hidden_size + 3 * widest)
         activations = sched.max_num_scheduled_tokens * per_token
         activations += sched.max_num_seqs * spec.vocab_size * (4 + esize)
-        margin = 512 << 20
-        budget = min(total * cache.gpu_memory_utilization - (total - free), free) - activations - margin
-        pages = int(budget // per_page)
-        if pages < 2:
-            raise RuntimeError(
-                f"not enough device memory for a KV cache: {free / 2**30:.1f} GiB free, "
-                f"{activations / 2**30:.2f} GiB of step buffers, {per_page} bytes per page")
-        return min(pages, useful)
+        budget = min(total * cache.gpu_memory_utilization - (total - free), free) - activations - (512 << 20)
+        return int(budget // max(self.bytes_per_page(), 1))
 
     # ---------------------------------------------------------------------- requests
     def add_request(self, request_id: str, sampling_params: SamplingParams, *,

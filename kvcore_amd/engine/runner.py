@@ -112,15 +112,11 @@ class ModelRunner:
             raise ValueError("page_size and num_pages must give one value per cache group")
         self.poison_pages = poison_pages
 
-        self.groups: list[CacheGroupView] = []
-        for gs, size, pages in zip(model.cache_groups, self.page_sizes, self.num_pages):
+        for gs, size in zip(model.cache_groups, self.page_sizes):
             if gs.need.page_size is not None and gs.need.page_size != size:
                 raise ValueError(f"a cache group wants pages of {gs.need.page_size} tokens, got {size}")
-            kv = torch.empty((gs.num_planes, 2, pages, gs.need.num_kv_heads, size, gs.need.head_dim),
-                             dtype=gs.need.dtype or self.dtype, device=self.device)
-            table = torch.zeros((max_num_seqs, -(-max_model_len // size)), dtype=torch.int32,
-                                device=self.device)
-            self.groups.append(CacheGroupView(kv, table, size, gs.need.window))
+        self.groups: list[CacheGroupView] = []
+        self._allocate_cache()
         # every part learns the sizes it will run at and may refuse them now, with a message,
         # rather than in the middle of a generation
         for call in model.calls:
@@ -193,6 +189,37 @@ class ModelRunner:
             self._graph_warm.clear()
             self._graph_pool = None  # the pool goes with its last graph
 
+    # -------------------------------------------------------------------- the cache
+    def _allocate_cache(self) -> None:
+        """Storage and block table of every cache group, as the groups' needs describe them:
+        a tensor ``[entries, pages, page_size * elements a token]`` per plane of the need."""
+        self.groups = []
+        for gs, size, pages in zip(self.model.cache_groups, self.page_sizes, self.num_pages):
+            dtype = gs.need.dtype or self.dtype
+            storage = [torch.empty((gs.num_planes, pages, size * elems), dtype=dtype, device=self.device)
+                       for elems in gs.need.token_elems()]
+            table = torch.zeros((self.max_num_seqs, -(-self.max_model_len // size)), dtype=torch.int32,
+                                device=self.device)
+            self.groups.append(CacheGroupView(storage, table, size, gs.need.window))
+
+    def resize_cache(self, num_pages: int | Sequence[int]) -> None:
+        """Give the cache back and allocate it anew with ``num_pages`` pages (a value per
+        group, the null page counted).  What the cache held is gone: for an engine that has
+        run its profile steps on a small cache and now knows how many pages fit.  Graphs are
+        dropped (they hold the old addresses), every slot is forgotten."""
+        n_groups = len(self.model.cache_groups)
+        self.num_pages = [num_pages] * n_groups if isinstance(num_pages, int) else list(num_pages)
+        if len(self.num_pages) != n_groups:
+            raise ValueError("num_pages must give one value per cache group")
+        torch.cuda.synchronize(self.device)
+        self._drop_graphs()
+        self.groups = []  # the old storage goes before the new one comes
+        torch.cuda.empty_cache()
+        self._allocate_cache()
+        self._slot_owner = [None] * self.max_num_seqs
+        self._slot_synced = [[0] * n_groups for _ in range(self.max_num_seqs)]
+        self._slot_released = [[0] * n_groups for _ in range(self.max_num_seqs)]
+
     # -------------------------------------------------------------------- bookkeeping
     def forget(self, slot: int) -> None:
         """A request left its slot.  The next owner's pages are synced from scratch."""
@@ -208,16 +235,18 @@ class ModelRunner:
             ids = [p for p in ids if p > 0]
             if ids:
                 dev = torch.tensor(ids, dtype=torch.int32, device=self.device)
-                ops.fill_pages(grp.kv, dev, len(ids), float("nan"))
+                for plane in grp.storage:
+                    ops.fill_pages(plane, dev, len(ids), float("nan"), page_axis=1)
 
     def fill_cache(self, value: float) -> None:
         """Overwrite every cache plane (tests fill with NaN so that a read outside a
         request's own slots shows in the logits)."""
         for g in self.groups:
-            g.kv.fill_(value)
+            for plane in g.storage:
+                plane.fill_(value)
 
     def cache_bytes(self) -> int:
-        return sum(g.kv.numel() * g.kv.element_size() for g in self.groups)
+        return sum(p.numel() * p.element_size() for g in self.groups for p in g.storage)
 
     def _table_updates(self, entries: Sequence[StepEntry]) -> list[list[int]]:
         """Per group, flat triples (slot, index, page) that bring the device tables up to
@@ -394,7 +423,8 @@ class ModelRunner:
                 triples = self._meta_dev[off:off + 3 * count]
                 ops.table_update(self.groups[g].table, triples, count)
                 if self.poison_pages:  # the pages listed for the first time: third of each triple
-                    ops.fill_pages(self.groups[g].kv, triples[2:], count, float("nan"), stride=3)
+                    for plane in self.groups[g].storage:
+                        ops.fill_pages(plane, triples[2:], count, float("nan"), stride=3, page_axis=1)
 
         ids = [e.request_id for e in entries]
         if bucket:
@@ -498,7 +528,7 @@ def describe_model(model: DecoderModel) -> str:
     return json.dumps({
         "layers": len(spec.layers), "schedule": len(spec.resolved_schedule()),
         "hidden": spec.hidden_size, "vocab": spec.vocab_size,
-        "cache_groups": [(g.need.num_kv_heads, g.need.head_dim, g.need.window, g.num_planes)
+        "cache_groups": [(g.need.planes, g.need.window, g.num_planes)
                          for g in model.cache_groups],
         "param_bytes": model.num_param_bytes(),
     })

@@ -40,7 +40,9 @@ def llama_spec(config: LlamaConfig) -> ModelSpec:
             mixer=attention,
             ffn=ffn,
             norms={"input_layernorm": norm, "post_attention_layernorm": norm},
-            block=PartSpec("prenorm", {"mixer_name": "self_attn", "ffn_name": "mlp"}),
+            block=PartSpec("prenorm", {"mixer_name": "self_attn", "ffn_name": "mlp",
+                                       "input_norm": "input_layernorm",
+                                       "post_norm": "post_attention_layernorm"}),
             position=0,
         )
         for i in range(config.num_hidden_layers)

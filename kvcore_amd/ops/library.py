@@ -166,17 +166,23 @@ def logits_finish(logits: torch.Tensor, bias: torch.Tensor | None = None, soft_c
                                     float(scale), _stream()), "kvc_logits_finish")
 
 
-def fill_pages(storage: torch.Tensor, pages: torch.Tensor, n: int, value: float, stride: int = 1) -> None:
-    """``storage`` is a cache group's ``[..., num_pages, kv_heads, page_size, head_dim]``
-    (contiguous, float32 or bfloat16); every element of the pages ``pages[i * stride]``,
-    ``i < n`` (int32 on the device), in all leading planes becomes ``value`` (0 or NaN as a
+def fill_pages(storage: torch.Tensor, pages: torch.Tensor, n: int, value: float, stride: int = 1,
+               page_axis: int = -4) -> None:
+    """``storage`` is cache memory whose axis ``page_axis`` counts pages, everything behind it
+    being one page and everything before it planes (a cache group's ``[entries, pages, elements
+    a page]`` with ``page_axis=1``; by default ``[..., pages, kv_heads, page_size, head_dim]``);
+    contiguous, float32 or bfloat16.  Every element of the pages ``pages[i * stride]``,
+    ``i < n`` (int32 on the device), in all planes becomes ``value`` (0 or NaN as a
     rule); the null page is skipped."""
-    if storage.dim() < 4 or not storage.is_contiguous():
-        raise KernelError("fill_pages: storage must be contiguous [..., pages, heads, page_size, d]")
+    axis = page_axis if page_axis >= 0 else storage.dim() + page_axis
+    if not 0 <= axis < storage.dim() - 1 or not storage.is_contiguous():
+        raise KernelError("fill_pages: storage must be contiguous [..., pages, a page...]")
     if n > 0 and pages.numel() < (n - 1) * stride + 1:
         raise KernelError("fill_pages: page list too short")
-    num_pages = storage.shape[-4]
-    page_elems = storage.shape[-3] * storage.shape[-2] * storage.shape[-1]
+    num_pages = storage.shape[axis]
+    page_elems = 1
+    for size in storage.shape[axis + 1:]:
+        page_elems *= size
     outer = storage.numel() // (num_pages * page_elems)
     esize = storage.element_size()
     probe = torch.tensor([value], dtype=storage.dtype)
@@ -818,13 +824,13 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
         return
     M, K = x.shape
     N = w.shape[0]
-    skinny_ok = _skinny_operands_ok(x, w)
-    # measured on MI355X (N x K of 4096..128256 x 4096..14336): the weight-streaming kernel
-    # wins up to 8 rows everywhere, up to 16 rows unless K or N is very large and up to 32 rows
-    # for small matrices
-    if skinny_ok and (M <= 8 or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)
-                      or (M <= 32 and K <= 4096 and N <= 4096)):
+    kernel = choose_product(M, N, K, few_rows_ok=_skinny_operands_ok(x, w),
+                            shared_rows_ok=mid_operands_ok(x, w) and out.stride(1) == 1)
+    if kernel == "few rows":
         gemm_skinny_bf16(out, x, w, bias)
+        return
+    if kernel == "shared rows":
+        gemm_mid(out, x, w, bias, mode=0)
         return
     if out.dtype == torch.float32:
         # the vendor product with float32 sums stored as they are (no rounding to bfloat16)
@@ -840,6 +846,27 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
         torch.mm(x, w.t(), out=out)
     else:
         torch.addmm(bias, x, w.t(), out=out)
+
+
+def choose_product(M: int, N: int, K: int, *, few_rows_ok: bool = True, shared_rows_ok: bool = True) -> str:
+    """Which kernel multiplies ``M`` rows of bfloat16 by an ``[N, K]`` matrix when nothing is
+    folded into the product: ``"few rows"`` (``gemm_skinny_bf16``: every wave streams its own
+    weight rows), ``"shared rows"`` (``gemm_mid``: the waves of a block share the rows through
+    LDS) or ``"vendor"`` (the vendor's product through torch).  The one place where row counts
+    and matrix sizes decide this; parts do not.  Measured on an MI355X with N x K from 4096 x
+    4096 to 128256 x 4096 and 8192 x 28672: the few-row kernel wins up to 8 rows everywhere,
+    up to 12 rows unless K is very long, up to 16 rows unless the output is as wide as a
+    vocabulary, and up to 32 rows for small matrices; from 17 to 64 rows the shared-row
+    kernel wins for outputs as wide as a vocabulary (215 against 231 us at 64 rows of 128256
+    x 4096) and the vendor's product is as fast or faster otherwise, as it is beyond 64 rows.
+    The flags say whether the operands' alignment and strides allow each kernel."""
+    if few_rows_ok and M <= SKINNY_MAX_ROWS and (
+            M <= 8 or (M <= 12 and K <= 8192) or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)
+            or (M <= 32 and K <= 4096 and N <= 4096)):
+        return "few rows"
+    if shared_rows_ok and SKINNY_PREFERRED_ROWS < M <= MID_ROWS and N >= 65536:
+        return "shared rows"
+    return "vendor"
 
 
 def table_update(table: torch.Tensor, triples: torch.Tensor, n: int) -> None:

@@ -141,7 +141,7 @@ class PagedAttention(Mixer):
         return specs
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(self.num_kv_heads, self.head_dim, self.window, self.page_size)
+        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window, self.page_size)
 
     def check_limits(self, limits) -> None:
         """The decode kernel keeps the page ids of a split's key range in LDS; a block table
@@ -166,7 +166,10 @@ class PagedAttention(Mixer):
         ops.linear(qkv, x, p["qkv_proj.weight"], p.get("qkv_proj.bias"))
 
         group = ctx.groups[call.group_index]
-        k_cache, v_cache = group.planes(call.cache_index)
+        # K pages [kv_heads, page, d]; V pages [kv_heads, d, page]: the keys of a page lie
+        # side by side, which is how the matrix cores want the values
+        k_cache = group.plane(call.cache_index, 0, self.num_kv_heads, group.page_size, self.head_dim)
+        v_cache = group.plane(call.cache_index, 1, self.num_kv_heads, self.head_dim, group.page_size)
         rot = self.position.rotary(ctx) if self.position is not None else None
         if rot is None:
             cos = sin = ctx.buffers.get("rope_none", ctx.num_tokens, 0, torch.float32)

@@ -58,19 +58,46 @@ class ParamSpec:
 
 @dataclass(frozen=True)
 class CacheNeed:
-    """Paged memory that grows with the sequence: keys and values of ``num_kv_heads``
-    heads of ``head_dim``.  ``window`` 0 keeps every token, ``w > 0`` only the last
+    """Paged memory that grows with the sequence.  ``planes`` lists what the mixer keeps per
+    token, a shape for each plane: keys and values of 8 heads of 128 are ``((8, 128), (8,
+    128))`` (:meth:`keys_and_values`), one compressed vector of 512 is ``((512,),)``, keys and
+    values of different widths are two shapes that differ.  A page of a plane holds
+    ``page_size`` tokens' worth of that shape in one contiguous piece; how the tokens lie
+    inside the page is the mixer's own business (``CacheGroupView.plane`` hands out pages as
+    flat rows, the mixer views them).  ``window`` 0 keeps every token, ``w > 0`` only the last
     ``w`` (pages wholly behind the window are given back during the request).
     ``page_size``: tokens per page if the mixer's kernels want a size of their own (None: the
     engine's ``block_size``); ``dtype``: the cache's element type (None: the model's).  Mixers
     with equal needs share a cache group; a group has its own page size, page count, pool,
     storage and block table."""
 
-    num_kv_heads: int
-    head_dim: int
+    planes: tuple[tuple[int, ...], ...]
     window: int = 0
     page_size: int | None = None
     dtype: torch.dtype | None = None
+
+    def __post_init__(self) -> None:
+        planes = tuple(tuple(int(n) for n in shape) for shape in self.planes)
+        if not planes or any(not shape or min(shape) <= 0 for shape in planes):
+            raise ValueError(f"a cache need names at least one plane of positive sizes, got {self.planes!r}")
+        object.__setattr__(self, "planes", planes)
+
+    @classmethod
+    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int = 0,
+                        page_size: int | None = None, dtype: torch.dtype | None = None) -> "CacheNeed":
+        """Two planes of ``num_kv_heads`` heads of ``head_dim``: what attention keeps."""
+        shape = (num_kv_heads, head_dim)
+        return cls((shape, shape), window, page_size, dtype)
+
+    def token_elems(self) -> tuple[int, ...]:
+        """Elements that one token takes in each plane."""
+        out = []
+        for shape in self.planes:
+            n = 1
+            for size in shape:
+                n *= size
+            out.append(n)
+        return tuple(out)
 
 
 @dataclass(frozen=True)

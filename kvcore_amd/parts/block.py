@@ -19,29 +19,38 @@ class PreNormBlock(Block):
     """``r += delta; a = mixer(norm_in(r)); r += a; out = ffn(norm_post(r))``, the last
     sum left pending for the next block's first norm."""
 
-    NORM_NAMES = ("input_layernorm", "post_attention_layernorm")
-
     def __init__(self, *, mixer: Mixer, ffn: FeedForward, norms: dict[str, Norm],
-                 mixer_name: str = "self_attn", ffn_name: str = "mlp") -> None:
+                 mixer_name: str = "self_attn", ffn_name: str = "mlp",
+                 input_norm: str | None = None, post_norm: str | None = None) -> None:
+        """``input_norm`` and ``post_norm`` name the norm before the mixer and the norm before
+        the feed-forward among ``norms`` (they are also the norms' checkpoint sub-prefixes);
+        left out, they are the first and the second norm that the layer lists."""
         super().__init__(mixer=mixer, ffn=ffn, norms=norms)
-        missing = [n for n in self.NORM_NAMES if n not in norms]
-        if missing:
-            raise ValueError(f"pre-norm block needs norms {self.NORM_NAMES}, missing {missing}")
+        listed = list(norms)
+        if input_norm is None and listed:
+            input_norm = listed[0]
+        if post_norm is None:
+            post_norm = next((n for n in listed if n != input_norm), None)
+        missing = [n for n in (input_norm, post_norm) if n not in norms]
+        if missing or input_norm == post_norm:
+            raise ValueError(f"a pre-norm block needs two norms, one before the mixer and one before the "
+                             f"feed-forward; asked for {(input_norm, post_norm)}, given {listed}")
+        self.norm_names = (input_norm, post_norm)
         self.mixer_name = mixer_name
         self.ffn_name = ffn_name
 
     def children(self) -> dict[str, Part]:
         return {
-            self.NORM_NAMES[0]: self.norms[self.NORM_NAMES[0]],
+            self.norm_names[0]: self.norms[self.norm_names[0]],
             self.mixer_name: self.mixer,
-            self.NORM_NAMES[1]: self.norms[self.NORM_NAMES[1]],
+            self.norm_names[1]: self.norms[self.norm_names[1]],
             self.ffn_name: self.ffn,
         }
 
     def input_gain(self, scaled: bool = True):
         """The first norm as (gain, eps) if the block before may do its work: leaving scaled
         rows for this block's mixer to finish (``scaled``), or finishing it itself."""
-        gain = self.norms[self.NORM_NAMES[0]].as_gain()
+        gain = self.norms[self.norm_names[0]].as_gain()
         if scaled and not self.mixer.takes_scaled_rows:
             return None
         return gain
@@ -59,9 +68,9 @@ class PreNormBlock(Block):
             x = delta.data  # the block before did the first norm
         else:
             x = ctx.buf("block_x", residual.shape[1])
-            self.norms[self.NORM_NAMES[0]].forward_fused(x, residual, delta)
+            self.norms[self.norm_names[0]].forward_fused(x, residual, delta)
 
-        post = self.norms[self.NORM_NAMES[1]]
+        post = self.norms[self.norm_names[1]]
         gain = None
         if self.mixer.takes_sink and ((fold and self.ffn.takes_scaled_rows) or sums):
             gain = post.as_gain()

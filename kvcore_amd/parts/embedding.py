@@ -65,24 +65,9 @@ class LinearHead(Head):
             ops.logits_finish(logits, bias, self.soft_cap, self.logit_scale)
 
     def _product(self, logits: torch.Tensor, hidden_rows: torch.Tensor) -> None:
-        w = self.params["weight"]
-        if hidden_rows.dtype == torch.float32:
-            ops.linear(logits, hidden_rows, w)
-            return
-        S = hidden_rows.shape[0]
-        # Every branch stores the float32 sums unrounded, so a request's logits do not change
-        # their rounding with the number of rows beside it.  Measured at 128256 x 4096: the
-        # few-row kernel wins up to 12 rows, the kernel that shares the rows through LDS from
-        # 17 to 64 (215 against 231 us at 64 rows), the vendor product in between and beyond.
-        if ops.skinny_operands_ok(hidden_rows, w) and (
-                S <= 12 or (S <= ops.SKINNY_PREFERRED_ROWS and self.vocab_size < 65536)):
-            ops.gemm_skinny_bf16(logits, hidden_rows, w)
-            return
-        if ops.SKINNY_PREFERRED_ROWS < S <= ops.MID_ROWS and ops.mid_operands_ok(hidden_rows, w) \
-                and logits.stride(1) == 1:
-            ops.gemm_mid(logits, hidden_rows, w, mode=0)
-            return
-        ops.linear(logits, hidden_rows, w)  # the vendor product, float32 out
+        """Every kernel that ``ops.linear`` may choose stores the float32 sums unrounded, so a
+        request's logits do not change their rounding with the number of rows beside it."""
+        ops.linear(logits, hidden_rows, self.params["weight"])
 
 
 OutputHead = LinearHead

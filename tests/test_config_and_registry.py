@@ -122,6 +122,12 @@ def test_engine_config_validation():
         SchedulerConfig(max_num_seqs=0)
     with pytest.raises(ValueError):
         SchedulerConfig(long_prefill_token_threshold=-1)
+    with pytest.raises(ValueError):
+        SchedulerConfig(max_num_partial_prefills=0)
+    # unset, every request that has a slot may be in its prompt; set, the number stands
+    assert SchedulerConfig().max_num_partial_prefills == 8
+    assert SchedulerConfig(max_num_seqs=32).max_num_partial_prefills == 32
+    assert SchedulerConfig(max_num_seqs=32, max_num_partial_prefills=1).max_num_partial_prefills == 1
     cfg = KVCoreConfig(ModelConfig(model="x", dtype="bf16"))
     assert cfg.model_config.dtype == "bfloat16"
     # the attention backend is filled in when unset (config.py:170-192); the reference's own
@@ -131,3 +137,16 @@ def test_engine_config_validation():
         ModelConfig(model="x", attn_backend="triton_paged")
     assert (cfg.cache_config.block_size, cfg.scheduler_config.max_num_seqs,
             cfg.scheduler_config.max_num_scheduled_tokens) == (16, 8, 512)
+
+
+def test_a_cache_need_describes_its_planes():
+    from kvcore_amd.parts.base import CacheNeed
+
+    kv = CacheNeed.keys_and_values(8, 128, window=0, page_size=None)
+    assert kv.planes == ((8, 128), (8, 128)) and kv.token_elems() == (1024, 1024)
+    assert CacheNeed(((512,),)).token_elems() == (512,)
+    assert CacheNeed([[2, 3], [5]]) == CacheNeed(((2, 3), (5,)))  # lists become tuples: needs are keys
+    assert len({CacheNeed(((4, 16), (4, 16))), CacheNeed.keys_and_values(4, 16)}) == 1
+    for bad in ((), ((),), ((4, 0),)):
+        with pytest.raises(ValueError):
+            CacheNeed(bad)

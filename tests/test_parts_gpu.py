@@ -124,11 +124,14 @@ def test_attention_part_in_two_portions(dtype, window):
         "bias": True, "window": window}), position=pe)
     p = bind_random(attn, dtype, seed=3)
     assert attn.cache_need().window == window and attn.state_need() is None
-    kv = torch.full((2, 2, 9, nkv, page, d), float("nan"), dtype=dtype, device=DEV)
+    need = attn.cache_need()
+    assert need.planes == ((nkv, d), (nkv, d)) and need.token_elems() == (nkv * d, nkv * d)
+    # two schedule entries, nine pages, a plane for the keys and one for the values
+    storage = [torch.full((2, 9, page * n), float("nan"), dtype=dtype, device=DEV) for n in need.token_elems()]
     table = torch.zeros(3, 8, dtype=torch.int32, device=DEV)
     table[2, :5] = torch.tensor([4, 7, 1, 8, 2], dtype=torch.int32)
-    group = CacheGroupView(kv, table, page, window)
-    call = LayerCall(0, 0, 0, 1, True, None)  # plane 1 of the group
+    group = CacheGroupView(storage, table, page, window)
+    call = LayerCall(0, 0, 0, 1, True, None)  # entry 1 of the group
     x = (torch.randn(18, H)).to(dtype).to(DEV)
     outs = []
     for lo, hi in ((0, 11), (11, 18)):
@@ -153,7 +156,7 @@ def test_attention_part_in_two_portions(dtype, window):
     o = plain.causal_gqa_attention(q, k, v, 0.3, window=window or None)
     want = o.reshape(T, nh * d) @ w["a.o_proj.weight"].T + w["a.o_proj.bias"]
     assert torch.allclose(got, want, **tol(dtype))
-    assert torch.isnan(kv[0]).all()  # plane 0 was not this call's to write
+    assert all(torch.isnan(plane[0]).all() for plane in storage)  # entry 0 was not this call's to write
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -197,6 +200,7 @@ def test_prenorm_block_against_the_reference_arrangement():
     assert list(block.children()) == ["input_layernorm", "self_attn", "post_attention_layernorm", "mlp"]
     ctx = make_ctx(torch.float32, [0, 1], [0, 0], [0])
     residual = torch.randn(2, H, device=DEV)
+    residual2 = residual.clone()
     delta = torch.randn(2, H, device=DEV)
     r = residual.double().cpu() + delta.double().cpu()
     a = 2 * plain.rms_norm(r, gains["input_layernorm"], 1e-6)
@@ -207,6 +211,16 @@ def test_prenorm_block_against_the_reference_arrangement():
     assert torch.allclose(residual.double().cpu(), r2, atol=1e-5)
     with pytest.raises(ValueError, match="norms"):
         BLOCKS.build(PartSpec("prenorm"), mixer=Doubler(), ffn=Negate(), norms={})
+    # the norms' names (their checkpoint sub-prefixes) are the architecture's to choose
+    renamed = {"ln_2": norms["post_attention_layernorm"], "ln_1": norms["input_layernorm"]}
+    other = BLOCKS.build(PartSpec("prenorm", {"input_norm": "ln_1", "post_norm": "ln_2", "mixer_name": "mix",
+                                              "ffn_name": "ff"}), mixer=Doubler(), ffn=Negate(), norms=renamed)
+    assert list(other.children()) == ["ln_1", "mix", "ln_2", "ff"]
+    out2 = other.forward(delta, residual2, ctx, None)
+    assert torch.equal(out2, out)
+    with pytest.raises(ValueError, match="norms"):
+        BLOCKS.build(PartSpec("prenorm", {"input_norm": "ln_1", "post_norm": "ln_3"}), mixer=Doubler(),
+                     ffn=Negate(), norms=renamed)
 
 
 def test_head_part_scale_vector_of_the_reference():

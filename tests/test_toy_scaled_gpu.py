@@ -127,7 +127,9 @@ def test_scaled_embedding_head_options_and_a_second_page_size(tmp_path, dtype, o
     assert [g.need.page_size for g in model.cache_groups] == [32, None]
     assert [g.page_size for g in session.manager.groups] == [32, PAGE]
     assert [grp.page_size for grp in session.runner.groups] == [32, PAGE]
-    assert session.runner.groups[0].kv.shape[-2] == 32 and session.runner.groups[1].kv.shape[-2] == PAGE
+    for grp, spec, size in zip(session.runner.groups, model.cache_groups, (32, PAGE)):
+        need = spec.need
+        assert [p.shape[2] for p in grp.storage] == [size * n for n in need.token_elems()]
     assert session.runner.groups[0].table.shape[1] == 256 // 32
     assert session.runner.groups[1].table.shape[1] == 256 // PAGE
 
