@@ -22,6 +22,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
+
 #include <cstdlib>
 
 #include "attention_combine.h"
@@ -423,6 +425,7 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
     // that no instruction waits for the one before it.
     f32x4_t s[CT][kKeyBlocks];
     constexpr int GK = (CT == 1) ? 2 : 1;  // key blocks a group
+    static_assert(kKeyBlocks % GK == 0, "the key blocks of a tile must come in whole groups");
     bf16x8_t ka[2][GK][NC];
     auto read_keys = [&](int grp, bf16x8_t (&dst)[GK][NC]) {
 #pragma unroll
@@ -456,6 +459,9 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
     constexpr bool kEarlyValues = CT == 1;
     constexpr int GJ = NJ / (2 * CT);  // operand reads a group
     constexpr int NG = NJ / GJ;        // groups a pair of key blocks
+    static_assert(GJ > 0 && NJ % GJ == 0,
+                  "a head size whose column groups do not divide into whole read groups would "
+                  "leave columns of the output without their sums");
     bf16x8_t va[2][GJ];
     auto read_values = [&](int pr, int grp, bf16x8_t (&dst)[GJ]) {
 #pragma unroll
@@ -631,6 +637,10 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
   const int64_t wide = (8 % nkv == 0) ? static_cast<int64_t>((max_pairs + 8 / nkv - 1) / (8 / nkv)) * 8
                                       : (static_cast<int64_t>(max_pairs) * nkv + 7) / 8 * 8;
   if (wide > 0x7fffffff) return kvc_fail("kvc_prefill_attention: too many blocks");
+  char variant[64];
+  snprintf(variant, sizeof(variant), "prefill_attention_kernel<%d,%d,%d,%d>%s x%d", D, CT, KB, W,
+           single ? " one tile a block" : "", nsplit);
+  kvc_note_variant(kVariantPrefillAttention, variant);
   hipLaunchKernelGGL((prefill_attention_kernel<D, CT, KB, W>), dim3(static_cast<unsigned>(wide), 1, nsplit), dim3(W * 64),
                      lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                      q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, part_o,

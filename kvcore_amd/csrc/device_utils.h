@@ -98,3 +98,8 @@ int kvc_check_launch(const char* what);
 // Compute units of the current device (asked of the runtime once per device; 256, an MI355X's,
 // if it will not say).  Launch plans count blocks against this, not against a constant.
 int kvc_device_compute_units(void);
+// Kernel families that have several variants to choose from at launch.  The entry points note
+// which one they launched (kvc_note_variant), and kvc_last_variant() tells the caller's thread:
+// for tests and tuning that must know which code ran.
+enum { kVariantPrefillAttention = 0, kVariantRopeKvWrite = 1, kVariantDecodeAttention = 2, kVariantFamilies = 3 };
+void kvc_note_variant(int family, const char* name);

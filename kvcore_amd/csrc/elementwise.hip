@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
 #include <mutex>
 #include <string>
 
@@ -49,6 +50,18 @@ extern "C" int kvc_compute_units(void) { return kvc_device_compute_units(); }
 
 extern "C" const char* kvc_last_error(void) { return g_last_error.c_str(); }
 extern "C" int kvc_version(void) { return 1; }
+
+static thread_local char g_variants[kVariantFamilies][64];
+
+void kvc_note_variant(int family, const char* name) {
+  if (family < 0 || family >= kVariantFamilies) return;
+  snprintf(g_variants[family], sizeof(g_variants[family]), "%s", name);
+}
+
+extern "C" const char* kvc_last_variant(int family) {
+  if (family < 0 || family >= kVariantFamilies) return "";
+  return g_variants[family];
+}
 
 static inline hipStream_t S(kvc_stream s) { return reinterpret_cast<hipStream_t>(s); }
 
@@ -784,6 +797,7 @@ extern "C" int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const 
                    aligned16(qkv) && aligned16(k_cache) && aligned16(cos_tab) && aligned16(sin_tab);
   if (vec && T >= 16 && aligned16(v_cache)) {
     // steps of many tokens: eight tokens a block
+    kvc_note_variant(kVariantRopeKvWrite, "rope_kv_write_tile_kernel");
     KVC_DISPATCH_DTYPE(
         dtype, Tp,
         hipLaunchKernelGGL((rope_kv_write_tile_kernel<Tp>), dim3((T + 7) / 8), dim3(256), 0, S(stream),
@@ -791,6 +805,7 @@ extern "C" int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const 
                            static_cast<Tp*>(v_cache), cos_tab, sin_tab, rot_dim, kv_slot, T, nh, nkv, d,
                            page_size, write_kv, head_begin));
   } else if (vec) {
+    kvc_note_variant(kVariantRopeKvWrite, "rope_kv_write_kernel<8>");
     KVC_DISPATCH_DTYPE(
         dtype, Tp,
         hipLaunchKernelGGL((rope_kv_write_kernel<Tp, 8>), dim3(T), dim3(256), 0, S(stream),
@@ -798,6 +813,7 @@ extern "C" int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const 
                            static_cast<Tp*>(v_cache), cos_tab, sin_tab, rot_dim, interleaved,
                            kv_slot, nh, nkv, d, page_size, write_kv, head_begin));
   } else {
+    kvc_note_variant(kVariantRopeKvWrite, "rope_kv_write_kernel<1>");
     KVC_DISPATCH_DTYPE(
         dtype, Tp,
         hipLaunchKernelGGL((rope_kv_write_kernel<Tp, 1>), dim3(T), dim3(256), 0, S(stream),

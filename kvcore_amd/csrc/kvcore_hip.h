@@ -19,6 +19,11 @@ int kvc_version(void);
 // Compute units of the current device: what the launch plans of the attention kernels count
 // blocks against.
 int kvc_compute_units(void);
+// The variant that this thread's last launch of a kernel family took, as a short text such as
+// "prefill_attention_kernel<128,1,8,8> x1" (head size, column tiles, key blocks a tile, waves,
+// then the number of splits) or "rope_kv_write_tile_kernel"; "" if the family has not been
+// launched.  Families: 0 attention over portions of prompts, 1 rotation with the cache write.
+const char* kvc_last_variant(int family);
 
 // residual[t, :] = float(table[ids[t], :]) * scale; an id outside [0, V) gives a NaN row.
 int kvc_embed(float* residual, const void* table, const int32_t* ids, int T, int H, int V,

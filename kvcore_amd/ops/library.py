@@ -78,6 +78,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.kvc_version.restype = c_int
     lib.kvc_compute_units.restype = c_int
     lib.kvc_compute_units.argtypes = []
+    lib.kvc_last_variant.restype = ctypes.c_char_p
+    lib.kvc_last_variant.argtypes = [c_int]
     lib.kvc_argmax_static_capacity.restype = c_int
     lib.kvc_argmax_static_capacity.argtypes = []
 
@@ -334,6 +336,15 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
 
 def decode_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype: torch.dtype) -> bool:
     return bool(load().kvc_decode_attention_supported(nh, nkv, d, page_size, DTYPE_CODE.get(dtype, -1)))
+
+
+KERNEL_FAMILIES = {"prefill_attention": 0, "rope_kv_write": 1}
+
+
+def last_variant(family: str) -> str:
+    """Which variant of a kernel family this thread's last launch took (see the C header): for
+    tests that must know which code ran."""
+    return load().kvc_last_variant(KERNEL_FAMILIES[family]).decode()
 
 
 _COMPUTE_UNITS: int | None = None

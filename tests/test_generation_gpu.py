@@ -367,3 +367,101 @@ def test_the_engine_equals_a_replay_of_the_trace_its_scheduler_produced(folders,
         compared += logits.shape[0]
     assert compared >= sum(12 + i for i in range(4)) + 9
     assert session.manager.live_requests() == []
+
+
+def check_sampled(cfg, weights, prompt, tokens, params, *, tol, exact_filters):
+    """Every token must be what ``tests/plain/sampling.sample`` draws from the plain logits
+    of the same prefix with the request's options and its noise of (seed, index).  Where it is
+    another token, the two must tie within rounding: the engine's token survives the filters
+    (``exact_filters``: the plain filters as they are; otherwise a logit may miss the top-k
+    threshold or the top-p boundary by ``tol``) and its score is within ``tol`` of the best."""
+    ids = list(prompt)
+    T = params.temperature
+    for index, tok in enumerate(tokens):
+        logits = plain.llama_forward(cfg, weights, ids, dtype=torch.float64)[-1]
+        want = plain_sampling.sample(logits, temperature=T, top_k=params.top_k, top_p=params.top_p,
+                                     seed=params.seed, index=index)
+        if tok != want:
+            assert T >= 1e-5 or float(logits.max() - logits[tok]) <= tol, f"token {index}: not the largest logit"
+            if T >= 1e-5:
+                scaled = logits / T
+                top_p = None if params.top_p >= 1.0 else params.top_p
+                kept = plain_sampling.apply_top_k_top_p(scaled, params.top_k, top_p)
+                if not exact_filters and kept[tok] == -math.inf:
+                    # the weakest survivor's logit, and the engine's token no further below it than rounding
+                    weakest = kept[kept > -math.inf].min()
+                    assert float(weakest - scaled[tok]) <= tol / T, (
+                        f"token {index}: {tok} is filtered out by top_k={params.top_k} top_p={params.top_p}")
+                    kept = kept.clone()
+                    kept[tok] = scaled[tok]
+                assert kept[tok] > -math.inf, (
+                    f"token {index}: {tok} is filtered out by top_k={params.top_k} top_p={params.top_p}")
+                score = kept - torch.log(plain_sampling.exponential_noise(params.seed, index, logits.numel()))
+                gap = float(score.max() - score[tok])
+                assert gap <= tol / T, f"token {index}: engine chose {tok}, plain draws {want} (ahead by {gap:.2e})"
+        ids.append(tok)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 5e-5), ("bfloat16", 6e-2)])
+def test_every_sampling_option_in_one_batch(folders, dtype, tol):
+    """Five requests side by side, each with other options: greedy, temperature alone, top-k,
+    top-p, and both; seeded, prompts cut into portions, decode steps launched ahead.  The rows
+    of one sampling call carry different options, so an option packed into another's column,
+    or a row given its neighbour's options, draws other tokens than the plain sampler."""
+    from kvcore_amd import SamplingParams
+
+    folder, cfg, weights, page = folders["B"]
+    options = [
+        SamplingParams(max_tokens=24, temperature=0.0, seed=11, ignore_eos=True),
+        SamplingParams(max_tokens=24, temperature=0.8, seed=12, ignore_eos=True),
+        SamplingParams(max_tokens=24, temperature=1.0, top_k=5, seed=13, ignore_eos=True),
+        SamplingParams(max_tokens=24, temperature=1.3, top_p=0.5, seed=14, ignore_eos=True),
+        SamplingParams(max_tokens=24, temperature=0.7, top_k=40, top_p=0.9, seed=15, ignore_eos=True),
+    ]
+    prompts = [random_tokens(n, 384, seed=700 + n) for n in (5, 33, 18, 47, 26)]
+    engine = make_engine(folder, dtype, page, max_seqs=8, budget=40, partial=8, threshold=16, run_ahead=True)
+    reqs = [dict(request_id=f"o{i}", prompt_token_ids=p, sampling_params=sp)
+            for i, (p, sp) in enumerate(zip(prompts, options))]
+    outs = {o.request_id: o.output_token_ids for o in engine.generate(reqs)}
+    assert engine.engine_core.runner.graph_replays > 0
+    for i, (p, sp) in enumerate(zip(prompts, options)):
+        toks = outs[f"o{i}"]
+        assert len(toks) == 24
+        check_sampled(cfg, weights, p, toks, sp, tol=tol, exact_filters=dtype == "float32")
+    # the filters did filter: with top_k = 5 every token is among the five largest logits of
+    # its row, which unfiltered noise over 384 flat logits would almost never give
+    ids = list(prompts[2])
+    for tok in outs["o2"]:
+        logits = plain.llama_forward(cfg, weights, ids, dtype=torch.float64)[-1]
+        assert float(logits[tok]) >= float(logits.topk(5).values[-1]) - tol
+        ids.append(tok)
+    # the same requests one at a time draw the same tokens: a row's draw does not depend on
+    # the rows beside it
+    if dtype == "float32":
+        alone = make_engine(folder, dtype, page, max_seqs=1, budget=64, partial=1)
+        for i, req in enumerate(reqs):
+            assert alone.generate([req])[0].output_token_ids == outs[f"o{i}"]
+
+
+def test_command_line_top_k_and_top_p(folders, tmp_path):
+    folder, cfg, weights, page = folders["B"]
+    cmd = [sys.executable, str(REPO / "bin" / "kvcore_offline_batch"), "--model", str(folder),
+           "--dtype", "float32", "--block-size", str(page), "--prompt-lens", "9,21", "--max-tokens", "12",
+           "--seed", "6", "--temperature", "1.1", "--top-k", "7", "--top-p", "0.8",
+           "--max-num-seqs", "4", "--max-num-scheduled-tokens", "32", "--num-gpu-blocks", "64",
+           "--ignore-eos", "--log-level", "WARNING", "--no-log-file"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=240)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    import random
+
+    from kvcore_amd import SamplingParams
+
+    rng = random.Random(6)
+    prompts = [[rng.randrange(384) for _ in range(n)] for n in (9, 21)]
+    lines = [l for l in proc.stdout.splitlines() if l.startswith("token_ids=")]
+    assert len(lines) == 2
+    params = SamplingParams(max_tokens=12, temperature=1.1, top_k=7, top_p=0.8, seed=6, ignore_eos=True)
+    for prompt, line in zip(prompts, lines):
+        got = [int(x) for x in line.split("=", 1)[1].strip("()").split(",") if x.strip()]
+        assert len(got) == 12
+        check_sampled(cfg, weights, prompt, got, params, tol=5e-5, exact_filters=True)

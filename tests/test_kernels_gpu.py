@@ -122,7 +122,9 @@ def test_gemm_f32_is_true_float32_and_does_not_depend_on_the_batch(ops, M, N, K)
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 16, 64), (5, 100, 200), (8, 4096, 4096), (16, 130, 1032),
-                                   (17, 6144, 512), (33, 48, 14336), (64, 1000, 2048)])
+                                   (17, 6144, 512), (33, 48, 14336), (64, 1000, 2048),
+                                   # the longest sum and the widest output of the 70B shape
+                                   (8, 8192, 28672), (12, 57344, 8192)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_gemm_skinny_bf16(ops, M, N, K, out_dtype):
     a = rnd(M, K, dtype=torch.bfloat16, seed=1)
@@ -154,7 +156,9 @@ def test_gemm_skinny_bf16(ops, M, N, K, out_dtype):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 200, 512), (33, 64, 1024), (48, 1000, 1536), (64, 4104, 1024),
-                                   (5, 72, 512), (64, 16400, 512)])
+                                   (5, 72, 512), (64, 16400, 512),
+                                   # the longest sum and the widest output of the 70B shape
+                                   (40, 8192, 28672), (24, 57344, 8192)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_gemm_mid_bf16(ops, M, N, K, out_dtype):
     """The product for a few dozen rows, whose waves share the rows through LDS: at once, and
@@ -196,7 +200,7 @@ def test_gemm_mid_bf16(ops, M, N, K, out_dtype):
     assert torch.equal(wide_out[:, :N], outs[0]) and torch.all(wide_out[:, N:] == 0)
 
 
-@pytest.mark.parametrize("M,I,K", [(17, 72, 512), (40, 1000, 1024), (64, 8200, 512)])
+@pytest.mark.parametrize("M,I,K", [(17, 72, 512), (40, 1000, 1024), (64, 8200, 512), (40, 28672, 8192)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gemm_mid_silu_mul(ops, M, I, K, with_bias):
     x = rnd(M, K, dtype=torch.bfloat16, seed=1)

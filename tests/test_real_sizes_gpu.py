@@ -51,7 +51,7 @@ def logit_rms(expect):
     return float(torch.cat([e.flatten() for e in expect.values()]).pow(2).mean().sqrt())
 
 
-def compare_rounding_noise(got, expect, row_bound=0.015, peak=6.5):
+def compare_rounding_noise(got, expect, row_bound=0.015, peak=6.5, what="rows of 128256"):
     """The bfloat16 bound for rows of 128,256 logits.  The engine rounds activations to
     bfloat16 (2^-9 relative, 0.11% in the root mean square) at a dozen places per layer and
     once before the head, so a row of logits carries noise of about 1% of the logits' root
@@ -62,10 +62,22 @@ def compare_rounding_noise(got, expect, row_bound=0.015, peak=6.5):
     logits, whose largest error is 3 deviations; here it is stated as what it means: a row's
     error is at most ``row_bound`` = 1.5% of the logits' root mean square in the root mean
     square (a slice of K left out of one product, 32 of 4,096 terms, gives 9%), and no single
-    logit errs by more than ``peak`` = 6.5 times that bound (a wrong weight row gives 140%)."""
+    logit errs by more than ``peak`` = 6.5 times that bound (a wrong weight row gives 140%).
+
+    Rows of a few hundred logits (the two-layer models with a small vocabulary): a row's
+    error and the logits' root mean square are then each estimated from V samples and scatter
+    by 1/sqrt(2V) of themselves, so their ratio scatters by 1/sqrt(V) (5% at V = 384), and it
+    varies from row to row besides.  Measured over all 2,048 rows of a 2,048-token prompt at
+    these widths with V = 384: mean 1.28%, standard deviation 0.11%, largest 1.71%, the same
+    at every depth of context (the float32 engine agrees with the plain implementation to
+    1e-6 there, so this is rounding alone).  For rows of fewer than 10,000 logits a single
+    row may therefore exceed ``row_bound`` by 4/sqrt(V) of it (1.81% at V = 384; a slice of K
+    left out still misses it five times over), and the mean over all compared rows must keep
+    ``row_bound`` itself."""
     from tests import helpers
 
     assert got, "nothing was compared"
+    ratios = []
     for (rid, pos), row in sorted(got.items()):
         ref = expect[rid][pos]
         assert torch.isfinite(row).all(), f"non-finite logits at {rid}:{pos}"
@@ -73,14 +85,18 @@ def compare_rounding_noise(got, expect, row_bound=0.015, peak=6.5):
         err = row - ref
         row_err = float(err.pow(2).mean().sqrt())
         worst = float(err.abs().max())
-        helpers.note_error("torch.bfloat16 rows of 128256 (root mean square)", row_err / (row_bound * scale), row_err)
-        helpers.note_error("torch.bfloat16 rows of 128256 (largest)", worst / (peak * row_bound * scale), worst)
-        assert row_err <= row_bound * scale, (
+        allowed = row_bound * (1.0 + 4.0 / ref.numel() ** 0.5) if ref.numel() < 10000 else row_bound
+        ratios.append(row_err / scale)
+        helpers.note_error(f"torch.bfloat16 {what} (root mean square)", row_err / (allowed * scale), row_err)
+        helpers.note_error(f"torch.bfloat16 {what} (largest)", worst / (peak * row_bound * scale), worst)
+        assert row_err <= allowed * scale, (
             f"request {rid} position {pos}: the row's error is {row_err / scale:.2%} of the logits' "
             f"root mean square")
         assert worst <= peak * row_bound * scale, (
             f"request {rid} position {pos}: logit {int(err.abs().argmax())} differs by {worst:.3e} "
             f"({worst / scale:.1%} of the logits' root mean square)")
+    mean = sum(ratios) / len(ratios)
+    assert mean <= row_bound, f"the rows' errors are {mean:.2%} of the logits' root mean square on average"
 
 
 def test_float32_engine_under_every_cut(real):
