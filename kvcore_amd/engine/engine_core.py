@@ -85,6 +85,21 @@ def resolve_dtype(config: KVCoreConfig, model_json: Mapping[str, Any]) -> torch.
     return TORCH_DTYPES[name or "bfloat16"]
 
 
+def join_stop_token_ids(config_eos, model_dir, tokenizer_manager) -> set[int]:
+    """The ids that end a request: config.json's ``eos_token_id``, the tokenizer's, and those
+    of the folder's generation_config.json.  The reference joins the first two
+    (engine_core.py:209-217); the third is this engine's addition, on purpose: instruct
+    checkpoints of Llama 3 name their end-of-turn id only there, and without it a chat request
+    runs to its length cap.  A folder whose generation_config.json lists further ids therefore
+    stops on them here and would not in the reference."""
+    stop = set(config_eos)
+    if model_dir is not None:
+        stop |= set(read_generation_eos(model_dir))
+    if tokenizer_manager is not None:
+        stop |= tokenizer_manager.get_stop_token_ids()
+    return stop
+
+
 class EngineCore:
     def __init__(self, config: KVCoreConfig, *, model=None) -> None:
         self.config = config
@@ -138,13 +153,9 @@ class EngineCore:
         if model_json:
             self.tokenizer_manager = TokenizerManager.from_model_source(
                 config.model_config.tokenizer or config.model_config.model)
-        # stop ids: config.json's, generation_config.json's and the tokenizer's, joined
-        # (reference: engine_core.py:209-217 joins the tokenizer's and the config's)
-        self.stop_token_ids = set(model.spec.eos_token_ids)
-        if model_json:
-            self.stop_token_ids |= set(read_generation_eos(config.model_config.model))
-        if self.tokenizer_manager is not None:
-            self.stop_token_ids |= self.tokenizer_manager.get_stop_token_ids()
+        self.stop_token_ids = join_stop_token_ids(
+            model.spec.eos_token_ids, config.model_config.model if model_json else None,
+            self.tokenizer_manager)
         self._seeds: dict[str, int] = {}
         self.run_ahead = sched.decode_run_ahead and model.device.type == "cuda"
         self._in_flight: _Flight | None = None

@@ -135,8 +135,12 @@ def fill_random(out: torch.Tensor, seed: int, name: str, init: str) -> None:
 
 def init_random_weights(model: DecoderModel, seed: int) -> None:
     """Fill every parameter in place, checkpoint tensor by checkpoint tensor, on the model's
-    device: the same values that ``write_random_model`` stores for this seed (a matrix kept
-    in bfloat16 is the float32 draw rounded once, as a file of bfloat16 matrices holds it)."""
+    device, from the same float32 draws that ``write_random_model`` makes for this seed.  A
+    matrix kept in bfloat16 is the draw rounded once, as a folder of bfloat16 matrices holds
+    it, so a bfloat16 model filled here equals one loaded from that folder bit for bit.  A
+    float32 model keeps the draws unrounded: it equals a folder written with
+    ``dtype=torch.float32``, and differs by that one rounding from a float32 model that loads
+    a folder of bfloat16 matrices (the default of ``write_random_model``)."""
     for name, (bp, row, rows) in model.checkpoint_map().items():
         fill_random(bp.tensor.narrow(0, row, rows), seed, name, bp.spec.init)
     if model.device.type == "cuda":

@@ -81,6 +81,19 @@ def test_generation_config_adds_stop_ids(tmp_path):
     (tmp_path / "generation_config.json").write_text("{not json")
     with pytest.raises(ConfigError):
         read_generation_eos(tmp_path)
+    # the engine joins them with config.json's and the tokenizer's: a deliberate addition to the
+    # reference's join (engine_core.py:209-217), which knows only those two
+    from kvcore_amd.engine.engine_core import join_stop_token_ids
+
+    class Tokenizer:
+        def get_stop_token_ids(self):
+            return {7, 128001}
+
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": [128001, 128009]}))
+    assert join_stop_token_ids((128001,), tmp_path, None) == {128001, 128009}
+    assert join_stop_token_ids((128001,), tmp_path, Tokenizer()) == {7, 128001, 128009}
+    assert join_stop_token_ids((128001,), None, Tokenizer()) == {7, 128001}  # a model given, no folder read
+    assert join_stop_token_ids((), None, None) == set()
 
 
 def test_registry_key_is_the_architecture_name_with_model_type_as_fallback():

@@ -62,12 +62,19 @@ def test_static_argmax_two_calls_in_a_row(lib):
     small = _logits(5, 20000, seed=2)       # 3 chunks a row: reads less of the array than is dirty
     out_big = torch.full((37,), -7, dtype=torch.int32, device=DEV)
     out_small = torch.full((5,), -7, dtype=torch.int32, device=DEV)
+    # the first call on a device looks up the array's address (and may load the code object):
+    # that is set-up; what is measured is a call after it
+    warm = torch.full((5,), -7, dtype=torch.int32, device=DEV)
+    assert _static(lib, small, warm) == 0, lib.kvc_last_error()
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    # torch's counters see its own allocator only; the device's free memory sees every
+    # hipMalloc of the process, the library's included
+    before = torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0]
     assert _static(lib, big, out_big) == 0, lib.kvc_last_error()
     assert _static(lib, small, out_small) == 0, lib.kvc_last_error()
     torch.cuda.synchronize()
-    assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == before
+    after = torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0]
+    assert after == before
     assert torch.equal(out_big, _reference(lib, big))
     assert torch.equal(out_small, _reference(lib, small))
     assert out_big.tolist() == big.cpu().argmax(-1).tolist()
@@ -76,6 +83,36 @@ def test_static_argmax_two_calls_in_a_row(lib):
     out_big.fill_(-7)
     assert _static(lib, big, out_big) == 0, lib.kvc_last_error()
     assert torch.equal(out_big, _reference(lib, big))
+
+
+def test_static_argmax_inside_a_captured_graph(lib):
+    """The callers it is for: a stream under capture cannot allocate.  Both calls are recorded
+    into one graph (the address was looked up before, outside the capture) and every replay,
+    with eager work of the same entry point in between, gives what ``kvc_argmax`` gives."""
+    big = _logits(21, 128256, seed=5)
+    small = _logits(4, 20000, seed=6)
+    out_big = torch.full((21,), -7, dtype=torch.int32, device=DEV)
+    out_small = torch.full((4,), -7, dtype=torch.int32, device=DEV)
+    other = _logits(9, 50000, seed=7)
+    out_other = torch.full((9,), -7, dtype=torch.int32, device=DEV)
+    assert _static(lib, small, out_small) == 0, lib.kvc_last_error()  # set-up, outside the capture
+    want_big, want_small = _reference(lib, big), _reference(lib, small)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            assert _static(lib, big, out_big) == 0, lib.kvc_last_error()
+            assert _static(lib, small, out_small) == 0, lib.kvc_last_error()
+    for i in range(3):
+        out_big.fill_(-7)
+        out_small.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_big, want_big) and torch.equal(out_small, want_small), f"replay {i}"
+        assert _static(lib, other, out_other) == 0, lib.kvc_last_error()  # dirties the array in between
+        torch.cuda.synchronize()
+        assert out_other.tolist() == other.cpu().argmax(-1).tolist()
 
 
 def test_static_argmax_strided_and_short_rows(lib):
