@@ -246,6 +246,7 @@ def main() -> int:
                             SamplingParams, SchedulerConfig)
     from kvcore_amd.engine.engine_core import EngineCore
     from kvcore_amd.engine.runner import build_model
+    from kvcore_amd.ops import library as ops_library
 
     model_name, base_cfg = MODELS[args.model]
     cfg = dict(base_cfg)
@@ -348,32 +349,44 @@ def main() -> int:
             drain()
         return sorted(times[1:])[1]  # median of the three after the warm-up run
 
+    def context_engine(ctx_len, b):
+        """An engine whose requests may reach ``ctx_len`` tokens of context."""
+        room = ctx_len + 128
+        return make_engine(room, b, b * -(-room // args.page_size) + 1)
+
+    def context_line(ctx_len, b, eng, steps=32, warmup=4):
+        # every request stays below ctx_len for the whole run (requests whose prompts end
+        # first decode while the others' prompts run), so that no step of the timed
+        # region is the first of a longer length class and captures its graph there
+        ahead = -(-b * ctx_len // PREFILL_TOKENS) + 2 + warmup + steps + 8
+        return decode_line(b, steps, warmup, eng, ctx_len - ahead)
+
+    def first_token_run(n, eng, runs=3):
+        """Seconds to the first token of one ``n``-token prompt in portions of 2,048."""
+        times = []
+        for i in range(runs):
+            new_request(n, 1, eng)
+            torch.cuda.synchronize()
+            t_start = time.perf_counter()
+            while eng.has_unfinished_requests():
+                eng.step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t_start)
+        return min(times[1:])
+
     if args.sweep:
         for b in (1, 2, 4, 8, 9, 12, 16, 24, 32, 48, 64):
             print(json.dumps(decode_line(b, 48, 8)), flush=True)
         del engine
         for ctx_len, batches in ((8192, (1, 8)), (32768, (1, 8)), (131072, (1,))):
             for b in batches:
-                # every request stays below ctx_len for the whole run (requests whose prompts end
-                # first decode while the others' prompts run), so that no step of the timed
-                # region is the first of a longer length class and captures its graph there
-                room = ctx_len + 128
-                eng = make_engine(room, b, b * -(-room // args.page_size) + 1)
-                ahead = -(-b * ctx_len // PREFILL_TOKENS) + 2 + 4 + 32 + 8
-                print(json.dumps(decode_line(b, 32, 4, eng, ctx_len - ahead)), flush=True)
+                eng = context_engine(ctx_len, b)
+                print(json.dumps(context_line(ctx_len, b, eng)), flush=True)
                 del eng
                 torch.cuda.empty_cache()
         return 0
     if args.long_prompt:
-        times = []
-        for i in range(3):
-            new_request(args.long_prompt, 1)
-            torch.cuda.synchronize()
-            t_start = time.perf_counter()
-            drain()
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t_start)
-        sec = min(times[1:])
+        sec = first_token_run(args.long_prompt, engine)
         print(json.dumps({"workload": f"first token of a {args.long_prompt}-token prompt in portions of "
                                       f"{PREFILL_TOKENS}", "model": model_name, "dtype": args.dtype,
                           "ms": round(sec * 1e3, 2), "tokens_per_s": round(args.long_prompt / sec, 1),
@@ -410,6 +423,10 @@ def main() -> int:
                           "tokens_per_s": round(PREFILL_TOKENS / sec, 1),
                           "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / sec / PEAK_FLOPS[args.dtype], 4)}))
         return 0
+    # what a kernel that only reads, and one that only multiplies, reach on this chip: the
+    # second yardstick beside the data sheet's
+    peaks = ops_library.measure_peaks(device)
+    measured_hbm, measured_mfma = peaks["read_bytes_per_s"], peaks["mfma_bf16_flops_per_s"]
     value, sec_per_step, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
     bytes_step = weight_bytes_per_step(cfg, esize) + kv_bytes(cfg, args.batch, mean_ctx, esize)
     achieved = bytes_step / sec_per_step
@@ -429,7 +446,9 @@ def main() -> int:
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single-gpu",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4),
+                     "measured_read_peak": round(measured_hbm / 1e9, 1),
+                     "frac_of_measured": round(achieved / measured_hbm, 4)},
     }
     if check is not None:
         result["check"] = check
@@ -439,6 +458,9 @@ def main() -> int:
         result["prefill"] = {"value": round(PREFILL_TOKENS / sec, 1), "tokens": PREFILL_TOKENS,
                              "ms": round(sec * 1e3, 3),
                              "frac": round(flops / sec / PEAK_FLOPS[args.dtype], 4)}
+        if args.dtype == "bf16":
+            result["prefill"]["measured_mfma_peak_tflops"] = round(measured_mfma / 1e12, 1)
+            result["prefill"]["frac_of_measured"] = round(flops / sec / measured_mfma, 4)
         points = {}
         for b in (1, 16, 32, 64):
             steps = max(16, min(args.steps, 64))
@@ -446,6 +468,24 @@ def main() -> int:
             points[f"decode_b{b}"] = round(v, 2)
             need = weight_bytes_per_step(cfg, esize) + kv_bytes(cfg, b, ctx_b, esize)
             points[f"decode_b{b}_hbm_frac"] = round(need / sec_b / HBM_PEAK, 4)
+        if args.model != "70b":
+            # further sizes: decode with 8k and 32k tokens of context a request (a length class
+            # each), and the time to the first token of an 8,192-token prompt in portions of 2,048
+            del engine
+            torch.cuda.empty_cache()
+            for ctx_len, key in ((8192, "8k"), (32768, "32k")):
+                eng = context_engine(ctx_len, 8)
+                line = context_line(ctx_len, 8, eng, steps=24, warmup=4)
+                points[f"decode_b8_ctx{key}"] = line["tokens_per_s"]
+                points[f"decode_b8_ctx{key}_ms"] = line["ms_per_step"]
+                points[f"decode_b8_ctx{key}_hbm_frac"] = line["hbm_frac"]
+                if ctx_len == 8192:
+                    sec_first = first_token_run(8192, eng)
+                    points["first_token_8192_ms"] = round(sec_first * 1e3, 2)
+                    points["first_token_8192_frac"] = round(
+                        prefill_flops(cfg, 8192) / sec_first / PEAK_FLOPS[args.dtype], 4)
+                del eng
+                torch.cuda.empty_cache()
         result["points"] = points
     print(json.dumps(result), flush=True)
     return 0

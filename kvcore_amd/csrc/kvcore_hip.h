@@ -25,6 +25,15 @@ int kvc_compute_units(void);
 // launched.  Families: 0 attention over portions of prompts, 1 rotation with the cache write.
 const char* kvc_last_variant(int family);
 
+// Measurement only (peaks.hip).  kvc_peak_read: `blocks` blocks of 256 threads read `bytes` bytes
+// of `buffer` once with 16-byte loads and store nothing (`sink`: four bytes that are practically
+// never written); timed by the caller over buffers too large for the caches, it gives the read
+// bandwidth that a kernel can reach at all.  kvc_peak_mfma_bf16: every wave of `blocks` blocks
+// of four issues `rounds` x 4 independent 32x32x16 bfloat16 matrix instructions on operands in
+// registers (2 x 32 x 32 x 16 flops each) and stores one float a thread into `out`.
+int kvc_peak_read(const void* buffer, int64_t bytes, int blocks, void* sink, kvc_stream stream);
+int kvc_peak_mfma_bf16(float* out, int blocks, int rounds, kvc_stream stream);
+
 // residual[t, :] = float(table[ids[t], :]) * scale; an id outside [0, V) gives a NaN row.
 int kvc_embed(float* residual, const void* table, const int32_t* ids, int T, int H, int V,
               int dtype, float scale, kvc_stream stream);

@@ -68,6 +68,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_argmax_static": [P, P, I, I, L, P],
         "kvc_sample": [P, P, I, I, L, P, P, P, P, P, P, P, L, I, P],
         "kvc_sample_workspace_words": [I, I],
+        "kvc_peak_read": [P, L, I, P, P],
+        "kvc_peak_mfma_bf16": [P, I, I, P],
     }
     for name, argtypes in sigs.items():
         fn = getattr(lib, name)
@@ -345,6 +347,45 @@ def last_variant(family: str) -> str:
     """Which variant of a kernel family this thread's last launch took (see the C header): for
     tests that must know which code ran."""
     return load().kvc_last_variant(KERNEL_FAMILIES[family]).decode()
+
+
+def measure_peaks(device: str | torch.device = "cuda:0") -> dict[str, float]:
+    """What this chip gives a kernel that does nothing but read (bytes a second: 16-byte loads
+    over 1 GiB pieces of a 3 GiB buffer, so that no cache serves them, two blocks a compute
+    unit) and nothing but multiply on the matrix cores (bfloat16 flops a second, operands in
+    registers, four waves a SIMD).  Some 0.1 s.  The data sheet says 8 TB/s and 2.5 PFLOP/s."""
+    lib = load()
+    device = torch.device(device)
+    cus = compute_units()
+    piece = 1 << 30
+    buf = torch.empty(3 * piece, dtype=torch.uint8, device=device)
+    buf.fill_(1)
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def read(i: int) -> None:
+        _check(lib.kvc_peak_read(buf.data_ptr() + (i % 3) * piece, piece, 2 * cus, sink.data_ptr(), _stream()),
+               "kvc_peak_read")
+
+    for i in range(3):
+        read(i)
+    start.record()
+    for i in range(12):
+        read(i)
+    end.record()
+    end.synchronize()
+    read_rate = 12 * piece / (start.elapsed_time(end) * 1e-3)
+    del buf
+    blocks, rounds = 4 * cus, 8000
+    out = torch.empty(blocks * 256, dtype=torch.float32, device=device)
+    for _ in range(2):
+        _check(lib.kvc_peak_mfma_bf16(out.data_ptr(), blocks, 200, _stream()), "kvc_peak_mfma_bf16")
+    start.record()
+    _check(lib.kvc_peak_mfma_bf16(out.data_ptr(), blocks, rounds, _stream()), "kvc_peak_mfma_bf16")
+    end.record()
+    end.synchronize()
+    flops = blocks * 4 * rounds * 4 * 2.0 * 32 * 32 * 16
+    return {"read_bytes_per_s": read_rate, "mfma_bf16_flops_per_s": flops / (start.elapsed_time(end) * 1e-3)}
 
 
 _COMPUTE_UNITS: int | None = None

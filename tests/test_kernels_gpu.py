@@ -1318,3 +1318,12 @@ def test_prefill_attention_long_context_and_many_tokens(ops, nh, nkv, d, whole, 
         for h in (0, nh - 1):
             p = torch.softmax((k[:, h // g] @ qd[t, h]) * scale, dim=0)
             assert torch.allclose(got[t, h], p @ v[:, h // g], atol=1e-2, rtol=1e-2), (t, h)
+
+
+def test_measured_peaks_are_of_this_chips_order(ops):
+    """The benchmark's second yardstick: a kernel that only reads and one that only multiplies.
+    An MI355X's data sheet says 8 TB/s and 2.5 PFLOP/s; the kernels must come within a factor
+    of two of those and cannot exceed them."""
+    peaks = ops.measure_peaks(DEV)
+    assert 4e12 < peaks["read_bytes_per_s"] < 8.2e12, peaks
+    assert 1.25e15 < peaks["mfma_bf16_flops_per_s"] < 2.6e15, peaks
