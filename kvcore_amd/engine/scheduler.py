@@ -285,20 +285,22 @@ class Scheduler:
         order, one position further, the token itself being ``AHEAD_TOKEN`` (the caller
         takes it from where the device left the sampled one).  Only a step of single
         decoded tokens that holds every running request is continued, and only if nothing
-        waits that a free slot could take, no request reaches its length cap or the context limit with ``output``, no
-        cache group has a window, and every page the next position needs is free: in every
+        waits that a free slot could take, no request reaches its length cap or the context
+        limit with ``output``, and every page the next position needs is free: in every
         other case the answer is None and the caller goes the ordinary way (``update`` then
         ``schedule``), which decides what this method does not.  Pages are taken at once;
-        a request that ends after all gives them back with the rest of its pages.  The
-        requests themselves are not touched: ``update_from_outputs`` takes the planned step
-        as it takes any other, once it has taken ``output``."""
+        a request that ends after all gives them back with the rest of its pages.  A cache
+        group with a window gives back, also at once, the pages that ``output`` moves the
+        window past, in the order in which ``update_from_outputs`` would (all requests first,
+        then the new pages are taken): ``output`` has been launched, the planned step follows it
+        on the same stream, so whoever gets such a page writes it after ``output`` has read it.
+        The requests themselves are not touched: ``update_from_outputs`` takes the planned
+        step as it takes any other, once it has taken ``output``."""
         if not output.scheduled or output.preempted_req_ids:
             return None
         if self.waiting and self.kv_manager.has_free_slot():
             return None  # with every slot taken nobody can be admitted (``schedule``, pass 2)
         if len(output.scheduled) != len(self.running):
-            return None
-        if any(g.window > 0 for g in self.kv_manager.groups):
             return None
         for s, request in zip(output.scheduled, self.running):
             if s.request_id != request.request_id or len(s.token_ids) != 1 or not s.samples or s.is_new:
@@ -307,6 +309,9 @@ class Scheduler:
                 return None  # ends with ``output``
             if s.num_computed_tokens + 2 > self.max_model_len:
                 return None
+        if any(g.window > 0 for g in self.kv_manager.groups):
+            for s in output.scheduled:  # what ``update_from_outputs`` will find done already
+                self.kv_manager.release_behind_window(s.request_id, s.num_computed_tokens + 1)
         planned: list[ScheduledRequest] = []
         for s in output.scheduled:
             start = s.num_computed_tokens + 1
@@ -316,8 +321,8 @@ class Scheduler:
                 request_id=s.request_id, slot=s.slot, is_new=False, token_ids=(AHEAD_TOKEN,),
                 num_computed_tokens=start,
                 page_ids=tuple(tuple(p) for p in self.kv_manager.page_ids(s.request_id)),
-                released=s.released, samples=True, num_output_tokens=s.num_output_tokens + 1,
-                sampling_params=s.sampling_params))
+                released=tuple(self.kv_manager.released_counts(s.request_id)), samples=True,
+                num_output_tokens=s.num_output_tokens + 1, sampling_params=s.sampling_params))
         return SchedulerOutput(tuple(planned), {s.request_id: 1 for s in planned}, len(planned),
                                frozenset(), (), output.step_id + 1)
 

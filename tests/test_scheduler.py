@@ -347,6 +347,47 @@ def test_a_step_planned_ahead_is_the_step_that_would_have_been_scheduled():
     assert s.requests["a"].output_token_ids[-3:] == [10, 12, 14]
 
 
+@pytest.mark.parametrize("window", [0, 3, 4])
+def test_steps_planned_ahead_with_a_window_are_the_ordinary_steps(window):
+    """Two schedulers with the same requests, one planning ahead, one going the ordinary way:
+    step for step the same positions, the same page lists (pages that the window has passed
+    are given back and read 0) and the same counts of released entries, so the pools hand out
+    the same pages in the same order."""
+    config = SchedulerConfig(max_num_seqs=3, max_num_scheduled_tokens=16, max_num_partial_prefills=3)
+    # with a window a dozen pages serve for good; without one every token keeps its place
+    num_pages = 12 if window else 40
+    ahead = make_scheduler(config, num_pages=num_pages, page=2, max_len=40, window=window)
+    plain_way = make_scheduler(config, num_pages=num_pages, page=2, max_len=40, window=window)
+    for sch in (ahead, plain_way):
+        sch.add_request(make_request("a", [1, 2, 3, 4, 5], max_tokens=14))
+        sch.add_request(make_request("b", [6, 7], max_tokens=14))
+        sch.add_request(make_request("c", [8, 9, 10, 11, 12, 13, 14], max_tokens=14))
+        sch.update_from_outputs(sch.schedule(), {"a": 20, "b": 21, "c": 22})
+    out_a = ahead.schedule()
+    planned_steps = 0
+    for step in range(12):
+        out_b = plain_way.schedule()
+        assert [(x.request_id, x.num_computed_tokens, x.page_ids, x.released, x.num_output_tokens)
+                for x in out_a.scheduled] == \
+               [(x.request_id, x.num_computed_tokens, x.page_ids, x.released, x.num_output_tokens)
+                for x in out_b.scheduled], step
+        planned = ahead.plan_decode_ahead(out_a)
+        tokens = {rid: 30 + step for rid in "abc"}
+        ahead.update_from_outputs(out_a, tokens)
+        plain_way.update_from_outputs(out_b, tokens)
+        ahead.kv_manager.check()
+        assert ahead.kv_manager.num_free_pages() == plain_way.kv_manager.num_free_pages() or planned is not None
+        if planned is not None:
+            planned_steps += 1
+            out_a = planned
+        else:
+            out_a = ahead.schedule()
+    assert planned_steps >= 10
+    if window:
+        assert any(n > 0 for x in out_a.scheduled for n in x.released)  # the window did pass pages
+        assert any(0 in pages for x in out_a.scheduled for pages in x.page_ids)
+
+
 def test_nothing_is_planned_ahead_when_the_ordinary_way_has_something_to_decide():
     config = SchedulerConfig(max_num_seqs=4, max_num_scheduled_tokens=16, max_num_partial_prefills=4)
     # a request reaches its length cap with the step
@@ -376,11 +417,6 @@ def test_nothing_is_planned_ahead_when_the_ordinary_way_has_something_to_decide(
     s.update_from_outputs(s.schedule(), {"a": 10, "b": 11})
     out = s.schedule()  # a: position 3 (page 2 of 2), b: position 1; three pages are out
     assert s.kv_manager.num_free_pages() == [0] and s.plan_decode_ahead(out) is None
-    # a window gives pages back as a request goes
-    s = make_scheduler(config, num_pages=32, max_len=24, window=4)
-    s.add_request(make_request("a", [1, 2, 3], max_tokens=8))
-    s.update_from_outputs(s.schedule(), {"a": 10})
-    assert s.plan_decode_ahead(s.schedule()) is None
     # the context limit
     s = make_scheduler(config, num_pages=32, max_len=5)
     s.add_request(make_request("a", [1, 2, 3], max_tokens=2))
@@ -388,8 +424,9 @@ def test_nothing_is_planned_ahead_when_the_ordinary_way_has_something_to_decide(
     assert s.plan_decode_ahead(s.schedule()) is None
 
 
+@pytest.mark.parametrize("window", [0, 5])
 @pytest.mark.parametrize("seed", range(6))
-def test_running_ahead_gives_the_outputs_of_the_ordinary_way(seed):
+def test_running_ahead_gives_the_outputs_of_the_ordinary_way(seed, window):
     """Stop tokens at random places (a request that stops has been planned one step too far),
     length caps, arrivals while others decode, and a pool small enough to preempt."""
     rng = random.Random(seed)
@@ -403,7 +440,8 @@ def test_running_ahead_gives_the_outputs_of_the_ordinary_way(seed):
     results = []
     for ahead in (False, True):
         s = make_scheduler(SchedulerConfig(max_num_seqs=4, max_num_scheduled_tokens=8, max_num_partial_prefills=2),
-                           num_pages=rng.choice([14, 40]) if not results else results[0][2], page=2, max_len=24)
+                           num_pages=rng.choice([14, 40]) if not results else results[0][2], page=2, max_len=24,
+                           window=window)
         pool = s.kv_manager.pools[0].num_usable + 1
         arriving = {t: [make_request(*specs[i]) for i in ids] for t, ids in arrivals.items()}
         outputs, steps, stats = _drive(s, ahead=ahead, stop_at=stop_at, arrivals=arriving)
