@@ -280,7 +280,14 @@ def main() -> int:
             device_config=DeviceConfig(device=device),
         ), model=model)
 
-    engine = make_engine(max(CONTEXT_LEN, args.long_prompt + 16), max_seqs, max_seqs * pages_per_seq + 1)
+    # the 70b shape fills most of the device: its cache is what the engine's own profile steps
+    # find room for; the other shapes get what the runs below can use
+    context_len = 4096 if args.model == "70b" else CONTEXT_LEN  # what the baseline names for each shape
+    engine = make_engine(max(context_len, args.long_prompt + 16), max_seqs,
+                         None if args.model == "70b" else max_seqs * pages_per_seq + 1)
+    if engine.memory_profile is not None:
+        print(f"[bench] cache sized by the engine: {engine.num_pages} pages of {args.page_size} tokens "
+              f"({engine.runner.cache_bytes() / 2**30:.1f} GiB)", file=sys.stderr, flush=True)
     rng = random.Random(0)
     vocab = cfg["vocab_size"]
     counter = [0]
@@ -441,7 +448,7 @@ def main() -> int:
             "layers_full": full_layers, "hidden": cfg["hidden_size"],
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"],
-            "vocab": cfg["vocab_size"], "global_batch": args.batch, "seq_len": CONTEXT_LEN,
+            "vocab": cfg["vocab_size"], "global_batch": args.batch, "seq_len": context_len,
             "prompt_len": prompt_len, "new_tokens": NEW_TOKENS, "page_size": args.page_size,
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single-gpu",
         },
