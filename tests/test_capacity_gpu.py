@@ -100,3 +100,34 @@ def test_a_tiny_model_gets_what_its_slots_can_use(tmp_path):
         outs[pages] = {o.request_id: o.output_token_ids for o in engine.generate(reqs)}
         core.kv_manager.check()
     assert outs[None] == outs[300]
+
+
+def test_profile_steps_run_on_a_model_with_state_and_parts_that_are_not_graph_safe(tmp_path):
+    """The profile steps drive whatever the registry built: here the toy architecture with a
+    mixer that keeps state of its own and walks the requests on the host (no graphs), a layer
+    that runs twice and one that reads another's cache.  The engine sizes itself and then
+    generates what an engine with a given page count generates."""
+    from kvcore_amd import CacheConfig, KVCoreConfig, ModelConfig, SamplingParams, SchedulerConfig
+    from kvcore_amd.engine.llm_engine import LLMEngine
+    from kvcore_amd.weights.loader import write_random_model
+    from tests.helpers import random_tokens
+    from tests.test_toy_parts_gpu import TOY_CONFIG, register_toy
+
+    register_toy()
+    folder = write_random_model(tmp_path / "toy", TOY_CONFIG, seed=9)
+    outs = {}
+    for pages in (None, 64):
+        engine = LLMEngine(KVCoreConfig(
+            model_config=ModelConfig(model=str(folder), dtype="float32", max_model_len=96),
+            cache_config=CacheConfig(block_size=8, num_gpu_blocks=pages),
+            scheduler_config=SchedulerConfig(max_num_seqs=3, max_num_scheduled_tokens=24)))
+        core = engine.engine_core
+        assert not core.model.graph_safe()
+        if pages is None:
+            assert core.memory_profile is not None and core.num_pages == 3 * 12 + 1
+        reqs = [dict(request_id=f"t{i}", prompt_token_ids=random_tokens(n, 97, seed=40 + i),
+                     sampling_params=SamplingParams(max_tokens=7, temperature=0.0, ignore_eos=True))
+                for i, n in enumerate((30, 4, 19, 11))]
+        outs[pages] = {o.request_id: o.output_token_ids for o in engine.generate(reqs)}
+        core.kv_manager.check()
+    assert outs[None] == outs[64] and all(len(t) == 7 for t in outs[None].values())
