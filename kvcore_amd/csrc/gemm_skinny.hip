@@ -416,14 +416,23 @@ void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M
 
 // The launch shape is a function of N and K alone, so that a row's sums do not depend on
 // how many rows come with it.  Measured on MI355X at 1 to 16 rows: 4 waves along K; outputs
-// wider than 4096 want 32 weight rows a wave, narrower ones 16.
+// wider than 4096 want 32 weight rows a wave, narrower ones 16.  Row-major matrices whose rows
+// lie a multiple of 16 KB apart (K a multiple of 8192: the 70B shape's qkv, o and head) are
+// the exception: a wave's two row tiles are then two streams at a distance that maps to the
+// same memory channels, and 16 rows a wave read faster, with 8 waves along K at K = 8192
+// (10240 x 8192: 42.7 against 51.2 us; 8192 x 8192: 28.8 against 33.8; 16384 x 8192: 52.6
+// against 59.8; 8192 x 16384 with 4 waves: 55.1 against 61.5; 8192 x 12288 and 8192 x 28672
+// are faster as they were, 38.3 against 41.9 and 80.4 against 88.5).
 // KVC_SKINNY_RT / KVC_SKINNY_WAVES override the choice for tuning.
 // From a packed matrix a wave takes 16 rows whatever N is: its second 16 rows would be a
 // second stream 16 * K elements behind the first, and the two together read slower than one
 // (128256 x 4096: 199 against 172 us; 28672 x 4096: 50.5 against 40.6 us).
 inline void pick_shape(int N, int K, int packed, int* rt_out, int* waves_out) {
   int rt, waves;
-  if (N > 4096 && !packed) {
+  if (N > 4096 && !packed && K % 8192 == 0) {
+    rt = 1;
+    waves = (K <= 8192) ? 8 : 4;
+  } else if (N > 4096 && !packed) {
     rt = 2;
     waves = 4;
   } else {
