@@ -477,6 +477,7 @@ int dispatch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int 
 int dispatch_gated(bf16_t* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M, int N,
                    int K, int64_t lda, int64_t ldc, const SkinnyExtras& ex, int packed, hipStream_t stream) {
   int waves = 4;
+  if (const char* e = getenv("KVC_SKINNY_GATED_WAVES")) waves = atoi(e) == 2 ? 2 : 4;  // for tuning
   while (waves > 1 && K / waves < 128) waves /= 2;
   const int nt = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
   int k_per_wave = (K + waves - 1) / waves;
