@@ -726,8 +726,11 @@ _skinny_operands_ok = skinny_operands_ok
 
 
 def mid_slices_bound(N: int) -> int:
-    """The most slices along K that ``gemm_mid`` cuts a weight with ``N`` rows into."""
-    return min(64, -(-256 // -(-N // 64)))
+    """The most slices along K that ``gemm_mid`` cuts a weight with ``N`` rows into: blocks
+    enough for 256 compute units, a block owning 64 weight rows, or 128 from 16,384 rows on
+    (``plan_mid`` in csrc/gemm_mid.hip)."""
+    rows_a_block = 128 if N >= 16384 else 64
+    return min(64, -(-256 // -(-N // rows_a_block)))
 
 
 def mid_slices(N: int, K: int) -> int:

@@ -58,7 +58,7 @@ def test_row_counts_choose_how_norms_and_products_meet():
 def test_slices_along_k_stay_within_the_bound_a_block_reserves_for():
     from kvcore_amd.ops import library as ops
 
-    for N in (64, 200, 2048, 4096, 8192, 14336, 128256):
+    for N in (64, 200, 2048, 4096, 8192, 14336, 16384, 20000, 28672, 32768, 57344, 128256):
         bound = ops.mid_slices_bound(N)
         assert 1 <= bound <= 64
         for K in (512, 1024, 4096, 14336, 28672, 65536):
