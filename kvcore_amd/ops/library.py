@@ -380,12 +380,15 @@ def measure_peaks(device: str | torch.device = "cuda:0") -> dict[str, float]:
     out = torch.empty(blocks * 256, dtype=torch.float32, device=device)
     for _ in range(2):
         _check(lib.kvc_peak_mfma_bf16(out.data_ptr(), blocks, 200, _stream()), "kvc_peak_mfma_bf16")
-    start.record()
-    _check(lib.kvc_peak_mfma_bf16(out.data_ptr(), blocks, rounds, _stream()), "kvc_peak_mfma_bf16")
-    end.record()
-    end.synchronize()
     flops = blocks * 4 * rounds * 4 * 2.0 * 32 * 32 * 16
-    return {"read_bytes_per_s": read_rate, "mfma_bf16_flops_per_s": flops / (start.elapsed_time(end) * 1e-3)}
+    best = 0.0
+    for _ in range(4):  # the clock takes a few milliseconds to rise: the fastest run is the peak
+        start.record()
+        _check(lib.kvc_peak_mfma_bf16(out.data_ptr(), blocks, rounds, _stream()), "kvc_peak_mfma_bf16")
+        end.record()
+        end.synchronize()
+        best = max(best, flops / (start.elapsed_time(end) * 1e-3))
+    return {"read_bytes_per_s": read_rate, "mfma_bf16_flops_per_s": best}
 
 
 _COMPUTE_UNITS: int | None = None
