@@ -141,7 +141,7 @@ class EngineCore:
         self.num_pages = first_pages
         self.group_configs = first_groups
         if profiled:
-            self.num_pages = self._measure_num_pages(first_pages)
+            self.num_pages = self._measure_num_pages()
             self.group_configs = plan_groups([g.need for g in model.cache_groups], self.page_size, self.num_pages)
             self.runner.resize_cache([g.num_pages for g in self.group_configs])
         self.kv_manager = KVManager(self.group_configs, max_num_seqs=sched.max_num_seqs,
@@ -224,7 +224,7 @@ class EngineCore:
         for _ in range(3):
             sample_both_ways(runner.step(entries).logits)
 
-    def _measure_num_pages(self, profile_pages: int) -> int:
+    def _measure_num_pages(self) -> int:
         """How many pages fit, by measurement (reference: model_runner.py:696-768 runs a dummy
         forward at ``max_num_scheduled_tokens``, reads torch's peak and gives the cache what
         ``gpu_memory_utilization`` of the device leaves beside it).  Here the profile steps run
