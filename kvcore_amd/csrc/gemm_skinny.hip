@@ -429,16 +429,11 @@ void launch(OutT* C, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M
 // (128256 x 4096: 199 against 172 us; 28672 x 4096: 50.5 against 40.6 us).
 inline void pick_shape(int N, int K, int packed, int* rt_out, int* waves_out) {
   int rt, waves;
-  if (N > 4096 && !packed && K % 8192 == 0) {
-    rt = 1;
-    waves = (K <= 8192) ? 8 : 4;
-  } else if (N > 4096 && !packed) {
-    rt = 2;
-    waves = 4;
-  } else {
-    rt = 1;
-    waves = 4;
-  }
+  // the waves along K are the same for a matrix and its packed copy, so that both give the
+  // same sums in the same order
+  const bool aligned_rows = N > 4096 && K % 8192 == 0;
+  waves = (aligned_rows && K <= 8192) ? 8 : 4;
+  rt = (N > 4096 && !packed && !aligned_rows) ? 2 : 1;
   while (waves > 1 && K / waves < 128) waves /= 2;
   if (const char* e = getenv("KVC_SKINNY_RT")) rt = atoi(e);
   if (const char* e = getenv("KVC_SKINNY_WAVES")) waves = atoi(e);

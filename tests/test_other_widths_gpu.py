@@ -126,3 +126,37 @@ def test_one_layer_of_the_other_shapes(shape, dtype, monkeypatch):
         # rows shared through LDS, single tokens and portions on the matrix cores
         assert {"gemm_skinny_bf16", "gemm_mid", "_fused_skinny", "decode_attention", "prefill_attention"} <= ran, ran
     assert session.manager.live_requests() == []
+
+
+def test_partial_packing_takes_the_matrices_whose_rows_collide_and_changes_no_bit(tmp_path):
+    """A model that has no room for packed copies of all its matrices (the 70B shape on one
+    device) packs those whose rows lie a multiple of 16 KB apart, whole shapes at a time, the
+    small shapes first, within a budget.  One layer at the 70B widths with room for 320 MB: the
+    head (384 x 8192), o_proj (8192 x 8192) and qkv_proj (10240 x 8192) are packed, gate_up
+    (57344 x 8192) does not fit, down_proj (8192 x 28672, rows 56 KB apart) does not qualify.
+    The logits are the bits of the model without any packed copy, and of the one with all."""
+    from kvcore_amd.engine.runner import build_model
+    from kvcore_amd.weights.loader import write_random_model
+
+    cfg = SHAPES["70b"]
+    folder = write_random_model(tmp_path / "w70", cfg, seed=5, device="cuda:0")
+    tokens = random_tokens(40, cfg["vocab_size"], seed=9)
+    steps = [{"step": 0, "entries": [{"id": "r", "tokens": tokens[:30], "want": [29]}], "end": []}]
+    steps += [{"step": i + 1, "entries": [{"id": "r", "tokens": [tokens[30 + i]], "want": [0]}], "end": []}
+              for i in range(10)]
+    rows = {}
+    for mode in ("none", "partial", "all"):
+        model = build_model(folder, torch.bfloat16, "cuda:0", pack_weights={"none": False, "all": True}.get(mode))
+        if mode == "partial":
+            taken = model.pack_product_weights(None, budget=320 << 20)
+            packed = sorted(tuple(w.shape) for w in model.product_weights() if getattr(w, "kvc_packed", None) is not None)
+            assert packed == [(384, 8192), (8192, 8192), (10240, 8192)], packed
+            assert taken == 2 * (384 + 8192 + 10240) * 8192
+        else:
+            count = sum(getattr(w, "kvc_packed", None) is not None for w in model.product_weights())
+            assert count == (5 if mode == "all" else 0)
+        session = session_for(folder, torch.bfloat16, PAGE, max_tokens=64, model=model)
+        rows[mode] = collect(session, steps)
+    assert len(rows["none"]) == 11
+    for key, row in rows["none"].items():
+        assert torch.equal(row, rows["partial"][key]) and torch.equal(row, rows["all"][key]), key
