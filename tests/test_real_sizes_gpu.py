@@ -165,7 +165,8 @@ def test_bfloat16_engine_with_every_row_count(real, monkeypatch):
     assert len([w for w in model.product_weights() if getattr(w, "kvc_packed", None) is not None]) == 9
     n_req = 70
     # requests in each decode step; steps of single tokens run padded to the runner's batch
-    # buckets (72, 40, 16, 16, 8, 4, 4 rows), which is what the head's product sees
+    # buckets (72, 40, 14, 12, 8, 4, 4 rows: every size from 8 to 16 has one), which is what the
+    # head's product sees
     live_after = [70, 40, 14, 12, 8, 3, 3]
     seqs = {}
     for i in range(n_req):
@@ -222,6 +223,6 @@ def test_bfloat16_engine_with_every_row_count(real, monkeypatch):
     compare_rounding_noise(got, expect)
     seen = set(head_paths)
     rows_12 = sum(fed_0 for fed_0 in (4 + int(r[1:]) % 5 for r in ids[60:62]))
-    assert {("vendor", 72), ("rows through LDS", 40), ("vendor", 16), ("few rows", 8), ("few rows", 4),
-            ("rows through LDS", 60), ("few rows", rows_12)} <= seen, seen
+    assert {("vendor", 72), ("rows through LDS", 40), ("vendor", 14), ("few rows", 12), ("few rows", 8),
+            ("few rows", 4), ("rows through LDS", 60), ("few rows", rows_12)} <= seen, seen
     assert session.manager.live_requests() == []
