@@ -145,7 +145,14 @@ class PagedAttention(Mixer):
 
     def check_limits(self, limits) -> None:
         """The decode kernel keeps the page ids of a split's key range in LDS; a block table
-        too wide for that is refused here, when the engine is built, not in a decode step."""
+        too wide for that is refused here, when the engine is built, not in a decode step.
+        So is a cache in another dtype than the model's, which the attention kernels do not
+        read (a subclass that names one in its ``cache_need`` must bring kernels that do)."""
+        need = self.cache_need()
+        if need.dtype is not None and need.dtype != self.runtime.dtype:
+            raise ValueError(
+                f"{type(self).__name__} keeps its cache in {need.dtype} beside a model in "
+                f"{self.runtime.dtype}: the attention kernels read keys and values in the model's dtype")
         if self.runtime.dtype != torch.bfloat16 or not ops.decode_attention_supported(
                 self.num_heads, self.num_kv_heads, self.head_dim, limits.page_size, self.runtime.dtype):
             return

@@ -292,3 +292,26 @@ def test_attention_refuses_a_block_table_wider_than_its_decode_kernel_serves():
     # float32 runs the general kernel, which has no such limit
     attn.setup(Runtime(torch.float32, DEV))
     attn.check_limits(RunLimits(8, 512, (widest + 1) * 16, 16, widest + 1))
+
+
+def test_attention_refuses_a_cache_in_another_dtype_when_it_is_built():
+    """``CacheNeed.dtype`` lets a mixer keep its cache in a dtype of its own; the attention
+    kernels read the model's, so a subclass that only changes the need is told so when the
+    runner is built, not by a kernel in its first step."""
+    from kvcore_amd.parts.attention import PagedAttention
+    from kvcore_amd.parts.base import CacheNeed, RunLimits, Runtime
+
+    class FloatCache(PagedAttention):
+        def cache_need(self):
+            return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, dtype=torch.float32)
+
+    args = dict(hidden_size=64, num_heads=4, num_kv_heads=2, head_dim=16, scale=0.25)
+    attn = FloatCache(**args)
+    attn.setup(Runtime(torch.bfloat16, DEV))
+    with pytest.raises(ValueError, match="keeps its cache in torch.float32"):
+        attn.check_limits(RunLimits(8, 512, 256, 16, 16))
+    attn.setup(Runtime(torch.float32, DEV))
+    attn.check_limits(RunLimits(8, 512, 256, 16, 16))
+    plain_attn = PagedAttention(**args)
+    plain_attn.setup(Runtime(torch.bfloat16, DEV))
+    plain_attn.check_limits(RunLimits(8, 512, 256, 16, 16))
