@@ -4,6 +4,8 @@ be fastest, and a kernel whose operands do not fit is never chosen."""
 
 from __future__ import annotations
 
+import pytest
+
 from kvcore_amd.ops.library import choose_product
 
 
@@ -26,3 +28,20 @@ def test_a_kernel_that_cannot_take_the_operands_is_not_chosen():
     assert choose_product(4, 4096, 4096, few_rows_ok=False) == "vendor"
     assert choose_product(40, 128256, 4096, shared_rows_ok=False) == "vendor"
     assert choose_product(40, 128256, 4096, few_rows_ok=False) == "shared rows"
+
+
+@pytest.mark.parametrize("limit", [1, 3, 6, 8, 11, 16, 20, 64, 100, 200, 1024])
+def test_decode_graph_sizes(limit):
+    """The batch sizes at which steps of single tokens are captured: rising, ending at the
+    engine's limit, every size from 8 to 16 (a padded row costs the few-row products what a
+    live one does), and never more than twice the live requests beyond one."""
+    from kvcore_amd.engine.runner import _decode_buckets
+
+    sizes = _decode_buckets(limit)
+    assert sizes == sorted(set(sizes)) and sizes[0] == 1 and sizes[-1] == limit
+    assert all(b in sizes for b in range(8, min(limit, 16) + 1))
+    for live in range(1, limit + 1):
+        padded = next(b for b in sizes if b >= live)
+        assert padded <= limit and padded < 2 * live + (live == 1)
+        if live > 16:
+            assert padded - live < 32
