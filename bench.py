@@ -265,7 +265,7 @@ def main() -> int:
     print(f"[bench] model built in {time.perf_counter() - t0:.1f} s, "
           f"{model.num_param_bytes() / 2**30:.2f} GiB", file=sys.stderr, flush=True)
 
-    max_seqs = 64
+    max_seqs = max(64, args.batch)  # request slots of the engine: every request of the batch decodes in every step
     pages_per_seq = -(-(PREFILL_TOKENS + NEW_TOKENS + prompt_len) // args.page_size)
     if args.long_prompt:
         max_seqs, pages_per_seq = 2, -(-(args.long_prompt + 16) // args.page_size)
@@ -385,6 +385,12 @@ def main() -> int:
         for b in (1, 2, 4, 8, 9, 12, 16, 24, 32, 48, 64):
             print(json.dumps(decode_line(b, 48, 8)), flush=True)
         del engine
+        torch.cuda.empty_cache()
+        eng = make_engine(context_len, 256, 256 * pages_per_seq + 1)
+        for b in (96, 128, 256):
+            print(json.dumps(decode_line(b, 32, 4, eng)), flush=True)
+        del eng
+        torch.cuda.empty_cache()
         for ctx_len, batches in ((8192, (1, 8)), (32768, (1, 8)), (131072, (1,))):
             for b in batches:
                 eng = context_engine(ctx_len, b)

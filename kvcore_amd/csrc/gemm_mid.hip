@@ -1,4 +1,4 @@
-// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for up to 64 rows of bfloat16 (used from 9 on),
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for up to 128 rows of bfloat16 (used from 17 on),
 // float32 sums: the decode step of a few dozen requests.  The weight matrix is still read
 // once from HBM, but the activations are no longer small beside a wave's share of it, so the
 // waves of a block share them through LDS instead of each reading its own copy from the cache.
@@ -42,6 +42,7 @@ constexpr int kRowElems = kChunk + 8;   // padded against bank conflicts
 constexpr int kStages = 4;              // steps of weights in flight per wave, the current one included
 constexpr int kRound = 64 * kStages;    // a slice of K is whole rounds of this many
 constexpr int kKMultiple = 512;         // what callers are promised: K is a multiple of this
+constexpr int kMaxRows = 128;           // rows of A: up to eight 16-row tiles a wave
 static_assert(kKMultiple % kRound == 0, "every K that is accepted must be whole rounds");
 
 template <int WAVES, int RT, int NT, bool GATED, typename OutT>
@@ -319,7 +320,10 @@ int dispatch_mid(OutT* C, float* partial, const bf16_t* A, const bf16_t* W, cons
     case 1: KVC_MID(W_, RT_, 1); break;                       \
     case 2: KVC_MID(W_, RT_, 2); break;                       \
     case 3: KVC_MID(W_, RT_, 3); break;                       \
-    default: KVC_MID(W_, RT_, 4); break;                      \
+    case 4: KVC_MID(W_, RT_, 4); break;                       \
+    case 5:                                                   \
+    case 6: KVC_MID(W_, RT_, 6); break;                       \
+    default: KVC_MID(W_, RT_, 8); break;                      \
   }
   if constexpr (GATED) {
     switch (p.waves) {
@@ -340,8 +344,8 @@ int dispatch_mid(OutT* C, float* partial, const bf16_t* A, const bf16_t* W, cons
 }
 
 int check_mid(const void* A, const void* W, int M, int N, int K, int64_t lda, int64_t ldc) {
-  if (M < 0 || M > 64 || N <= 0 || K <= 0 || lda < K || ldc < N)
-    return kvc_fail("kvc_gemm_mid_bf16: bad sizes (1 to 64 rows)");
+  if (M < 0 || M > kMaxRows || N <= 0 || K <= 0 || lda < K || ldc < N)
+    return kvc_fail("kvc_gemm_mid_bf16: bad sizes (1 to 128 rows)");
   if (K % kKMultiple || lda % 8)
     return kvc_fail("kvc_gemm_mid_bf16: K must be a multiple of 512 and the row stride of 8");
   if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15))

@@ -157,8 +157,11 @@ def test_gemm_skinny_bf16(ops, M, N, K, out_dtype):
 
 @pytest.mark.parametrize("M,N,K", [(17, 200, 512), (33, 64, 1024), (48, 1000, 1536), (64, 4104, 1024),
                                    (5, 72, 512), (64, 16400, 512),
+                                   # more than four tiles of 16 rows: five and six run as six, seven and eight as eight
+                                   (65, 200, 1024), (81, 4104, 512), (96, 1000, 1536), (100, 16400, 512),
+                                   (128, 4096, 4096), (113, 72, 512),
                                    # the longest sum and the widest output of the 70B shape
-                                   (40, 8192, 28672), (24, 57344, 8192)])
+                                   (40, 8192, 28672), (24, 57344, 8192), (128, 8192, 28672)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_gemm_mid_bf16(ops, M, N, K, out_dtype):
     """The product for a few dozen rows, whose waves share the rows through LDS: at once, and
@@ -200,7 +203,8 @@ def test_gemm_mid_bf16(ops, M, N, K, out_dtype):
     assert torch.equal(wide_out[:, :N], outs[0]) and torch.all(wide_out[:, N:] == 0)
 
 
-@pytest.mark.parametrize("M,I,K", [(17, 72, 512), (40, 1000, 1024), (64, 8200, 512), (40, 28672, 8192)])
+@pytest.mark.parametrize("M,I,K", [(17, 72, 512), (40, 1000, 1024), (64, 8200, 512), (40, 28672, 8192),
+                                   (72, 1000, 1024), (96, 8200, 512), (128, 14336, 4096), (127, 72, 512)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gemm_mid_silu_mul(ops, M, I, K, with_bias):
     x = rnd(M, K, dtype=torch.bfloat16, seed=1)
@@ -225,10 +229,10 @@ def test_gemm_mid_refuses_what_it_does_not_take(ops):
     w = rnd(64, 520, dtype=torch.bfloat16)
     with pytest.raises(ops.KernelError, match="multiple of 512"):
         ops.gemm_mid(torch.empty(20, 64, dtype=torch.bfloat16, device=DEV), a, w)
-    a = rnd(65, 512, dtype=torch.bfloat16)
+    a = rnd(129, 512, dtype=torch.bfloat16)
     w = rnd(64, 512, dtype=torch.bfloat16)
-    with pytest.raises(ops.KernelError, match="1 to 64 rows"):
-        ops.gemm_mid(torch.empty(65, 64, dtype=torch.bfloat16, device=DEV), a, w)
+    with pytest.raises(ops.KernelError, match="1 to 128 rows"):
+        ops.gemm_mid(torch.empty(129, 64, dtype=torch.bfloat16, device=DEV), a, w)
 
 
 @pytest.mark.parametrize("T,H,slices,with_bias", [(17, 64, 1, False), (40, 1000, 3, True), (64, 4096, 4, False),
