@@ -1,4 +1,4 @@
-// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for up to 128 rows of bfloat16 (used from 17 on),
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for up to 192 rows of bfloat16 (used from 17 on),
 // float32 sums: the decode step of a few dozen requests.  The weight matrix is still read
 // once from HBM, but the activations are no longer small beside a wave's share of it, so the
 // waves of a block share them through LDS instead of each reading its own copy from the cache.
@@ -42,7 +42,7 @@ constexpr int kRowElems = kChunk + 8;   // padded against bank conflicts
 constexpr int kStages = 4;              // steps of weights in flight per wave, the current one included
 constexpr int kRound = 64 * kStages;    // a slice of K is whole rounds of this many
 constexpr int kKMultiple = 512;         // what callers are promised: K is a multiple of this
-constexpr int kMaxRows = 128;           // rows of A: up to eight 16-row tiles a wave
+constexpr int kMaxRows = 192;           // rows of A: up to twelve 16-row tiles a wave (sixteen were measured slower than the vendor's product)
 static_assert(kKMultiple % kRound == 0, "every K that is accepted must be whole rounds");
 
 template <int WAVES, int RT, int NT, bool GATED, typename OutT>
@@ -132,16 +132,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mid_kernel(
   auto mma_step = [&](int stage, int buf, int part) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      bf16x8_t b[NT];
+      // the tiles of A four at a time: with many tiles, all of them at once cost registers
+      constexpr int G = NT < 4 ? NT : 4;
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        b[nt] = *reinterpret_cast<const bf16x8_t*>(
-            &a_lds[buf][(nt * 16 + col) * kRowElems + part * 64 + h * 32 + 8 * quad]);
+      for (int n0 = 0; n0 < NT; n0 += G) {
+        bf16x8_t b[G];
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
+        for (int j = 0; j < G; ++j)
+          if (n0 + j < NT)
+            b[j] = *reinterpret_cast<const bf16x8_t*>(
+                &a_lds[buf][((n0 + j) * 16 + col) * kRowElems + part * 64 + h * 32 + 8 * quad]);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wbuf[stage][rt][h], b[nt], acc[rt][nt], 0, 0, 0);
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int j = 0; j < G; ++j)
+            if (n0 + j < NT)
+              acc[rt][n0 + j] =
+                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(wbuf[stage][rt][h], b[j], acc[rt][n0 + j], 0, 0, 0);
+      }
     }
   };
 
@@ -313,6 +321,10 @@ template <bool GATED, typename OutT>
 int dispatch_mid(OutT* C, float* partial, const bf16_t* A, const bf16_t* W, const bf16_t* bias, int M,
                  int N, int K, int64_t lda, int64_t ldc, const MidPlan& p, hipStream_t stream) {
   const int nt = (M + 15) / 16;
+  // with more than eight tiles of rows a block of two waves would hold a chunk of A in more
+  // registers than there are: four waves then (the slices along K, and with them the order of
+  // every sum, stay as planned)
+  const int waves = nt > 8 ? 4 : p.waves;
 #define KVC_MID(W_, RT_, NT_) \
   launch_mid<W_, RT_, NT_, GATED, OutT>(C, partial, A, W, bias, M, N, K, lda, ldc, p, stream)
 #define KVC_MID_NT(W_, RT_)                                   \
@@ -323,15 +335,20 @@ int dispatch_mid(OutT* C, float* partial, const bf16_t* A, const bf16_t* W, cons
     case 4: KVC_MID(W_, RT_, 4); break;                       \
     case 5:                                                   \
     case 6: KVC_MID(W_, RT_, 6); break;                       \
-    default: KVC_MID(W_, RT_, 8); break;                      \
+    case 7:                                                   \
+    case 8: KVC_MID(W_, RT_, 8); break;                       \
+    case 9:                                                   \
+    case 10:                                                  \
+    case 11:                                                  \
+    default: KVC_MID(W_, RT_, 12); break;                     \
   }
   if constexpr (GATED) {
-    switch (p.waves) {
+    switch (waves) {
       case 2: KVC_MID_NT(2, 2); break;
       default: KVC_MID_NT(4, 2); break;
     }
   } else {
-    switch (p.waves * 10 + p.rt) {
+    switch (waves * 10 + p.rt) {
       case 21: KVC_MID_NT(2, 1); break;
       case 22: KVC_MID_NT(2, 2); break;
       case 42: KVC_MID_NT(4, 2); break;
@@ -345,7 +362,7 @@ int dispatch_mid(OutT* C, float* partial, const bf16_t* A, const bf16_t* W, cons
 
 int check_mid(const void* A, const void* W, int M, int N, int K, int64_t lda, int64_t ldc) {
   if (M < 0 || M > kMaxRows || N <= 0 || K <= 0 || lda < K || ldc < N)
-    return kvc_fail("kvc_gemm_mid_bf16: bad sizes (1 to 128 rows)");
+    return kvc_fail("kvc_gemm_mid_bf16: bad sizes (1 to 192 rows)");
   if (K % kKMultiple || lda % 8)
     return kvc_fail("kvc_gemm_mid_bf16: K must be a multiple of 512 and the row stride of 8");
   if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15))

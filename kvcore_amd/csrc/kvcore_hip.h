@@ -170,7 +170,7 @@ int kvc_prefill_attention(void* out, const void* q, int64_t q_stride, const void
 int kvc_gemm_f32(float* C, const float* A, const float* W, const float* bias, int M, int N,
                  int K, int64_t lda, int64_t ldc, kvc_stream stream);
 
-// The same product for 17 to 128 rows, where the waves of a block share the rows of A through
+// The same product for 17 to 192 rows, where the waves of a block share the rows of A through
 // LDS (K a multiple of 512).  mode 0: C = A W^T (+ bias), float32 (out_dtype 0) or bfloat16
 // (1).  mode 1: C[M, N] = silu(A Wg^T + bg) * (A Wu^T + bu) in bfloat16, W [2N, K] holding Wg
 // then Wu.  mode 2: narrow outputs are cut along K into kvc_gemm_mid_slices(N, K) slices and

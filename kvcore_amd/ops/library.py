@@ -628,7 +628,7 @@ class ResidualSink:
     eps: float
     out: torch.Tensor
     ss_parts: torch.Tensor | None
-    # for steps of 17 to 128 rows: float32 room for the partial sums of a product cut along K
+    # for steps of 17 to 192 rows: float32 room for the partial sums of a product cut along K
     # (``mid_slices_bound(N) * T * N`` values); the sink then finishes the norm itself and
     # ``out`` receives the normalised rows
     slices: torch.Tensor | None = None
@@ -637,16 +637,17 @@ class ResidualSink:
 @dataclass
 class NormedRows:
     """Rows that a :class:`ResidualSink` has already added into the residual and normalised:
-    what ``linear`` returns for a sink that carries a workspace (steps of 17 to 128 rows)."""
+    what ``linear`` returns for a sink that carries a workspace (steps of 17 to 192 rows)."""
 
     data: torch.Tensor
 
 
-# The most rows the kernel that shares its rows through LDS takes (eight tiles of 16 a wave).
+# The most rows the kernel that shares its rows through LDS takes (twelve tiles of 16 a wave).
 # Measured on the 8B shape against the vendor's products with a norm kernel between them, a
 # whole decode step: 72 rows 5.93 against 6.66 ms, 96 rows 6.53 against 7.72, 128 rows 7.57
-# against 8.63.
-MID_ROWS = 128
+# against 8.63, 160 rows 9.37 against 9.79, 192 rows 10.12 against 11.35; with sixteen tiles a
+# wave 256 rows took 12.86 against 11.11, so the vendor's product has them.
+MID_ROWS = 192
 
 
 # Up to here the few-row kernel with the norms folded in is the fastest.  Measured at 16 rows
@@ -663,7 +664,7 @@ def rows_fusable(num_rows: int, dtype: torch.dtype) -> bool:
 
 def rows_sinkable(num_rows: int, dtype: torch.dtype) -> bool:
     """Whether a step of ``num_rows`` tokens sends the products before its norms into a
-    :class:`ResidualSink` that finishes the norm itself: 17 to 128 rows."""
+    :class:`ResidualSink` that finishes the norm itself: 17 to 192 rows."""
     return dtype == torch.bfloat16 and FOLD_ROWS < num_rows <= MID_ROWS
 
 
@@ -753,7 +754,7 @@ def mid_operands_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 def gemm_mid(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
              *, mode: int = 0, partial: torch.Tensor | None = None) -> None:
-    """The weight-streaming product for up to 128 rows of bfloat16 whose waves share the rows
+    """The weight-streaming product for up to 192 rows of bfloat16 whose waves share the rows
     through LDS, the faster one from 9 rows on (see the C header for the
     modes: 0 plain, 1 ``silu(gate) * up``, 2 partial sums of slices along K only, 3 plain
     with slices and a kernel that sums them)."""
@@ -797,7 +798,7 @@ def add_slices_rmsnorm(out: torch.Tensor, residual: torch.Tensor, partial: torch
 
 
 def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None) -> NormedRows:
-    """A product of 17 to 128 rows into a sink: partial sums of slices along K, then one kernel
+    """A product of 17 to 192 rows into a sink: partial sums of slices along K, then one kernel
     that adds them into the residual and normalises.  Shapes the weight-streaming kernel does
     not take run the vendor product into the same workspace first."""
     M, K = x.shape
@@ -854,7 +855,7 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and x.is_cuda and FOLD_ROWS < M <= MID_ROWS and mid_operands_ok(x, w)
             and out.stride(1) == 1):
-        # 17 to 128 rows: the waves of a block share the rows through LDS
+        # 17 to 192 rows: the waves of a block share the rows through LDS
         gemm_mid(out, x, w, bias, mode=1)
         return
     gate_up = scratch()
@@ -869,7 +870,7 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
     vendor matrix product through torch.  All sum in float32, and a float32 ``out`` receives
     the sums unrounded on either path.  With a :class:`ScaledRows` for ``x`` or a :class:`ResidualSink` for ``out``
     (few rows of bfloat16 only) the norm before or after the product is folded into it; a
-    sink returns the :class:`ScaledRows` it made, or, in a step of 17 to 128 rows, where it
+    sink returns the :class:`ScaledRows` it made, or, in a step of 17 to 192 rows, where it
     finishes the norm itself, :class:`NormedRows`."""
     if isinstance(out, ResidualSink) and out.slices is not None:
         if isinstance(x, ScaledRows):
@@ -918,9 +919,9 @@ def choose_product(M: int, N: int, K: int, *, few_rows_ok: bool = True, shared_r
     and matrix sizes decide this; parts do not.  Measured on an MI355X with N x K from 4096 x
     4096 to 128256 x 4096 and 8192 x 28672: the few-row kernel wins up to 8 rows everywhere,
     up to 12 rows unless K is very long, up to 16 rows unless the output is as wide as a
-    vocabulary, and up to 32 rows for small matrices; from 17 to 128 rows the shared-row
+    vocabulary, and up to 32 rows for small matrices; from 17 to 192 rows the shared-row
     kernel wins for outputs as wide as a vocabulary (215 against 231 us at 64 rows of 128256
-    x 4096) and the vendor's product is as fast or faster otherwise, as it is beyond 128 rows.
+    x 4096) and the vendor's product is as fast or faster otherwise, as it is beyond 192 rows.
     The flags say whether the operands' alignment and strides allow each kernel."""
     if few_rows_ok and M <= SKINNY_MAX_ROWS and (
             M <= 8 or (M <= 12 and K <= 8192) or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)

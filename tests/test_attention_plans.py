@@ -45,12 +45,12 @@ def test_row_counts_choose_how_norms_and_products_meet():
     from kvcore_amd.ops import library as ops
 
     bf16, f32 = torch.bfloat16, torch.float32
-    # the products do the norms' work up to 16 rows; from 17 to 128 a kernel of its own finishes them
+    # the products do the norms' work up to 16 rows; from 17 to 192 a kernel of its own finishes them
     assert ops.rows_fusable(1, bf16) and ops.rows_fusable(16, bf16)
     assert not ops.rows_fusable(17, bf16) and ops.rows_sinkable(17, bf16)
-    assert ops.rows_sinkable(128, bf16) and not ops.rows_sinkable(129, bf16)
+    assert ops.rows_sinkable(192, bf16) and not ops.rows_sinkable(193, bf16)
     # never both, and float32 neither
-    for rows in range(0, 140):
+    for rows in range(0, 200):
         assert not (ops.rows_fusable(rows, bf16) and ops.rows_sinkable(rows, bf16))
         assert not ops.rows_fusable(rows, f32) and not ops.rows_sinkable(rows, f32)
 

@@ -160,6 +160,8 @@ def test_gemm_skinny_bf16(ops, M, N, K, out_dtype):
                                    # more than four tiles of 16 rows: five and six run as six, seven and eight as eight
                                    (65, 200, 1024), (81, 4104, 512), (96, 1000, 1536), (100, 16400, 512),
                                    (128, 4096, 4096), (113, 72, 512),
+                                   # nine to twelve tiles run as twelve
+                                   (129, 200, 512), (192, 4096, 4096), (150, 1000, 1536), (192, 16400, 512), (177, 72, 1024),
                                    # the longest sum and the widest output of the 70B shape
                                    (40, 8192, 28672), (24, 57344, 8192), (128, 8192, 28672)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
@@ -204,7 +206,8 @@ def test_gemm_mid_bf16(ops, M, N, K, out_dtype):
 
 
 @pytest.mark.parametrize("M,I,K", [(17, 72, 512), (40, 1000, 1024), (64, 8200, 512), (40, 28672, 8192),
-                                   (72, 1000, 1024), (96, 8200, 512), (128, 14336, 4096), (127, 72, 512)])
+                                   (72, 1000, 1024), (96, 8200, 512), (128, 14336, 4096), (127, 72, 512),
+                                   (130, 1000, 512), (160, 8200, 1024), (192, 14336, 4096), (191, 72, 512)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gemm_mid_silu_mul(ops, M, I, K, with_bias):
     x = rnd(M, K, dtype=torch.bfloat16, seed=1)
@@ -229,10 +232,10 @@ def test_gemm_mid_refuses_what_it_does_not_take(ops):
     w = rnd(64, 520, dtype=torch.bfloat16)
     with pytest.raises(ops.KernelError, match="multiple of 512"):
         ops.gemm_mid(torch.empty(20, 64, dtype=torch.bfloat16, device=DEV), a, w)
-    a = rnd(129, 512, dtype=torch.bfloat16)
+    a = rnd(193, 512, dtype=torch.bfloat16)
     w = rnd(64, 512, dtype=torch.bfloat16)
-    with pytest.raises(ops.KernelError, match="1 to 128 rows"):
-        ops.gemm_mid(torch.empty(129, 64, dtype=torch.bfloat16, device=DEV), a, w)
+    with pytest.raises(ops.KernelError, match="1 to 192 rows"):
+        ops.gemm_mid(torch.empty(193, 64, dtype=torch.bfloat16, device=DEV), a, w)
 
 
 @pytest.mark.parametrize("T,H,slices,with_bias", [(17, 64, 1, False), (40, 1000, 3, True), (64, 4096, 4, False),
