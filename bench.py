@@ -385,18 +385,15 @@ def main() -> int:
         for b in (1, 2, 4, 8, 9, 12, 16, 24, 32, 48, 64):
             print(json.dumps(decode_line(b, 48, 8)), flush=True)
         del engine
-        torch.cuda.empty_cache()
-        eng = make_engine(context_len, 256, 256 * pages_per_seq + 1)
-        for b in (96, 128, 256):
-            print(json.dumps(decode_line(b, 32, 4, eng)), flush=True)
-        del eng
-        torch.cuda.empty_cache()
         for ctx_len, batches in ((8192, (1, 8)), (32768, (1, 8)), (131072, (1,))):
             for b in batches:
                 eng = context_engine(ctx_len, b)
                 print(json.dumps(context_line(ctx_len, b, eng)), flush=True)
                 del eng
                 torch.cuda.empty_cache()
+        eng = make_engine(context_len, 256, 256 * pages_per_seq + 1)
+        for b in (96, 128, 192, 256):
+            print(json.dumps(decode_line(b, 32, 4, eng)), flush=True)
         return 0
     if args.long_prompt:
         sec = first_token_run(args.long_prompt, engine)
