@@ -648,6 +648,18 @@ class NormedRows:
 # against 8.63, 160 rows 9.37 against 9.79, 192 rows 10.12 against 11.35; with sixteen tiles a
 # wave 256 rows took 12.86 against 11.11, so the vendor's product has them.
 MID_ROWS = 192
+# Which products gain beyond 64 rows, one by one against the vendor's (us at 96 / 128 / 192 rows,
+# packed weights): the narrow ones that are cut along K do (4096 x 14336: 33 / 45 / 64 against
+# 64 / 76 / 104; 4096 x 4096: 13 / 15 / 21 against 23 / 25 / 34; 8192 x 28672: 109 / 136 / 209
+# against 123 / 201 / 232); the gated one up to 128 rows (28672 x 4096: 54 / 67 / 83 against 53 /
+# 54 / 61 and an activation kernel of 8 to 12; in a whole step of 128 rows 7.64 against 7.74 ms,
+# of 192 rows 10.19 against 9.96); the head does not (128256 x 4096: 224 / 256 / 324 against
+# 226 / 233 / 254; no difference in a whole step).  Matrices without a packed copy are read row by row, which
+# the vendor's product does better from 65 rows on (a step of the 70B shape at 96 requests:
+# 40.8 ms against 43.6).
+MID_ROWS_UNPACKED = 64
+MID_ROWS_GATED = 128
+MID_ROWS_WIDE = 64
 
 
 # Up to here the few-row kernel with the norms folded in is the fastest.  Measured at 16 rows
@@ -812,7 +824,7 @@ def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.
     # measured: the vendor product is as fast or faster once the output is wide and K is not
     # long (8192 x 8192), and slower for narrow outputs and long K (8192 x 28672: 139 against
     # 107 us at 64 rows; 4096 x 4096: 19 against 12)
-    ours = N < 8192 or K > 8192
+    ours = (N < 8192 or K > 8192) and (M <= MID_ROWS_UNPACKED or bool(_streamed(w, N)[1]))
     if ours and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and mid_operands_ok(x, w) and N % 8 == 0:
         slices = mid_slices(N, K)
         if sink.slices.numel() < slices * M * N:
@@ -853,9 +865,9 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
             M, I, K, x.stride(0), out.stride(0), packed, _stream()), "kvc_gemm_skinny_silu_mul_bf16")
         return
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
-            and x.is_cuda and FOLD_ROWS < M <= MID_ROWS and mid_operands_ok(x, w)
-            and out.stride(1) == 1):
-        # 17 to 192 rows: the waves of a block share the rows through LDS
+            and x.is_cuda and mid_operands_ok(x, w) and out.stride(1) == 1
+            and FOLD_ROWS < M <= (MID_ROWS_GATED if _streamed(w, I)[1] else MID_ROWS_UNPACKED)):
+        # 17 to 128 rows: the waves of a block share the rows through LDS
         gemm_mid(out, x, w, bias, mode=1)
         return
     gate_up = scratch()
@@ -919,15 +931,15 @@ def choose_product(M: int, N: int, K: int, *, few_rows_ok: bool = True, shared_r
     and matrix sizes decide this; parts do not.  Measured on an MI355X with N x K from 4096 x
     4096 to 128256 x 4096 and 8192 x 28672: the few-row kernel wins up to 8 rows everywhere,
     up to 12 rows unless K is very long, up to 16 rows unless the output is as wide as a
-    vocabulary, and up to 32 rows for small matrices; from 17 to 192 rows the shared-row
+    vocabulary, and up to 32 rows for small matrices; from 17 to 64 rows the shared-row
     kernel wins for outputs as wide as a vocabulary (215 against 231 us at 64 rows of 128256
-    x 4096) and the vendor's product is as fast or faster otherwise, as it is beyond 192 rows.
+    x 4096) and the vendor's product is as fast or faster otherwise, as it is beyond 64 rows.
     The flags say whether the operands' alignment and strides allow each kernel."""
     if few_rows_ok and M <= SKINNY_MAX_ROWS and (
             M <= 8 or (M <= 12 and K <= 8192) or (M <= SKINNY_PREFERRED_ROWS and K <= 8192 and N < 65536)
             or (M <= 32 and K <= 4096 and N <= 4096)):
         return "few rows"
-    if shared_rows_ok and SKINNY_PREFERRED_ROWS < M <= MID_ROWS and N >= 65536:
+    if shared_rows_ok and SKINNY_PREFERRED_ROWS < M <= MID_ROWS_WIDE and N >= 65536:
         return "shared rows"
     return "vendor"
 

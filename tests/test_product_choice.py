@@ -14,12 +14,11 @@ def test_row_counts_and_sizes_choose_the_kernel():
     for N, K in (qkv_8b, down_8b, head, down_70b, o_1b):
         for M in (1, 2, 8):
             assert choose_product(M, N, K) == "few rows"
-        for M in (193, 512, 2048):
+        for M in (65, 512, 2048):
             assert choose_product(M, N, K) == "vendor"
     assert choose_product(12, *head) == "few rows" and choose_product(13, *head) == "vendor"
     assert choose_product(16, *head) == "vendor"
     assert choose_product(17, *head) == "shared rows" and choose_product(64, *head) == "shared rows"
-    assert choose_product(192, *head) == "shared rows" and choose_product(65, *qkv_8b) == "vendor"
     assert choose_product(16, *qkv_8b) == "few rows" and choose_product(17, *qkv_8b) == "vendor"
     assert choose_product(9, *down_8b) == "vendor" and choose_product(9, *down_70b) == "vendor"
     assert choose_product(32, *o_1b) == "few rows" and choose_product(33, *o_1b) == "vendor"
