@@ -656,8 +656,10 @@ MID_ROWS = 192
 # of 192 rows 10.19 against 9.96); the head does not (128256 x 4096: 224 / 256 / 324 against
 # 226 / 233 / 254; no difference in a whole step).  Matrices without a packed copy are read row by row, which
 # the vendor's product does better from 65 rows on (a step of the 70B shape at 96 requests:
-# 40.8 ms against 43.6).
+# 40.8 ms against 43.6) and up to 32 (24 requests: 30.4 against 32.7 ms, 32: 31.2 against 32.8;
+# 48: 39.2 against 36.3, 64: the same).
 MID_ROWS_UNPACKED = 64
+MID_ROWS_UNPACKED_FROM = 33
 MID_ROWS_GATED = 128
 MID_ROWS_WIDE = 64
 
@@ -666,6 +668,14 @@ MID_ROWS_WIDE = 64
 # against the kernels that share their rows through LDS: the 8B shape 4.13 against 4.45 ms a
 # step, the 70B shape 30.4 against 32.6, the 1B shape 1.13 against 1.11.
 FOLD_ROWS = 16
+
+
+def mid_rows_ok(num_rows: int, packed: bool, most: int) -> bool:
+    """Whether a product of ``num_rows`` rows by a matrix with or without a packed copy runs in
+    the kernel that shares its rows through LDS (``most``: the kind of product's own limit)."""
+    if packed:
+        return FOLD_ROWS < num_rows <= most
+    return MID_ROWS_UNPACKED_FROM <= num_rows <= min(most, MID_ROWS_UNPACKED)
 
 
 def rows_fusable(num_rows: int, dtype: torch.dtype) -> bool:
@@ -824,7 +834,7 @@ def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.
     # measured: the vendor product is as fast or faster once the output is wide and K is not
     # long (8192 x 8192), and slower for narrow outputs and long K (8192 x 28672: 139 against
     # 107 us at 64 rows; 4096 x 4096: 19 against 12)
-    ours = (N < 8192 or K > 8192) and (M <= MID_ROWS_UNPACKED or bool(_streamed(w, N)[1]))
+    ours = (N < 8192 or K > 8192) and mid_rows_ok(M, bool(_streamed(w, N)[1]), MID_ROWS)
     if ours and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and mid_operands_ok(x, w) and N % 8 == 0:
         slices = mid_slices(N, K)
         if sink.slices.numel() < slices * M * N:
@@ -866,7 +876,7 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
         return
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and x.is_cuda and mid_operands_ok(x, w) and out.stride(1) == 1
-            and FOLD_ROWS < M <= (MID_ROWS_GATED if _streamed(w, I)[1] else MID_ROWS_UNPACKED)):
+            and mid_rows_ok(M, bool(_streamed(w, I)[1]), MID_ROWS_GATED)):
         # 17 to 128 rows: the waves of a block share the rows through LDS
         gemm_mid(out, x, w, bias, mode=1)
         return

@@ -214,9 +214,9 @@ def test_gemm_mid_silu_mul(ops, M, I, K, with_bias):
     w = rnd(2 * I, K, dtype=torch.bfloat16, seed=2, scale=0.1)
     bias = rnd(2 * I, dtype=torch.bfloat16, seed=3) if with_bias else None
     out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
-    if M <= ops.MID_ROWS_UNPACKED:
+    if ops.mid_rows_ok(M, False, ops.MID_ROWS_GATED):
         ops.linear_silu_mul(out, x, w, bias, lambda: pytest.fail("the one-kernel form should have run"))
-    else:  # more rows take the one-kernel form only with a packed copy of the weights (tested below)
+    else:  # fewer or more rows take the one-kernel form only with a packed copy of the weights (tested below)
         ops.gemm_mid(out, x, w, bias, mode=1)
     # both factors rounded to bfloat16 first, as the two-kernel form stores them (the two
     # forms start their walks along K at different places, so not the same bits)
@@ -231,27 +231,27 @@ def test_gemm_mid_silu_mul(ops, M, I, K, with_bias):
 
 
 def test_beyond_64_rows_the_kernel_for_a_few_dozen_rows_runs_where_it_was_measured_faster(ops, monkeypatch):
-    """Packed weights: the gated product up to 128 rows, the products cut along K up to 192;
-    weights read row by row and the wide head go to the vendor's product from 65 rows on."""
+    """Packed weights: the gated product from 17 to 128 rows, the products cut along K up to
+    192; weights read row by row only from 33 to 64 rows, the vendor's product has the rest."""
     ran = []
     real_mid, real_mm = ops.gemm_mid, torch.mm
     monkeypatch.setattr(ops, "gemm_mid", lambda *a, **kw: (ran.append("mid"), real_mid(*a, **kw))[1])
     monkeypatch.setattr(torch, "mm", lambda *a, **kw: (ran.append("vendor"), real_mm(*a, **kw))[1])
-    I, K, H = 1024, 512, 512
+    I, K, H = 4096, 512, 512
     w_gate_up = (rnd(2 * I, K, dtype=torch.bfloat16, seed=2) * 0.1).contiguous()
     w_down = (rnd(H, I, dtype=torch.bfloat16, seed=3) * 0.1).contiguous()
     for packed in (False, True):
         if packed:
             ops.pack_weight(w_gate_up)
             ops.pack_weight(w_down)
-        for M, gated_ours, sliced_ours in ((64, True, True), (96, packed, packed), (128, packed, packed), (144, False, packed),
+        for M, gated_ours, sliced_ours in ((24, packed, packed), (33, True, True), (64, True, True), (96, packed, packed), (128, packed, packed), (144, False, packed),
                                            (192, False, packed), (200, False, False)):
             x = rnd(M, K, dtype=torch.bfloat16, seed=1)
             h = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
             scratch = torch.empty(M, 2 * I, dtype=torch.bfloat16, device=DEV)
             ran.clear()
             ops.linear_silu_mul(h, x, w_gate_up, None, lambda: scratch)
-            assert ran == (["mid"] if gated_ours else ["vendor"]), (packed, M, ran)
+            assert ran == (["mid"] if gated_ours else ["vendor"]), (packed, M, ran)  # (8192 x 512 is no matrix for the few-row kernel at 24 rows)
             want = torch.nn.functional.silu(x.double() @ w_gate_up[:I].double().T) * (x.double() @ w_gate_up[I:].double().T)
             assert torch.allclose(h.double(), want, atol=3e-2, rtol=3e-2)
             if M > ops.MID_ROWS:
@@ -262,7 +262,8 @@ def test_beyond_64_rows_the_kernel_for_a_few_dozen_rows_runs_where_it_was_measur
                                     None, torch.empty(ops.mid_slices_bound(H) * ops.MID_ROWS * H, device=DEV))
             ran.clear()
             ops.linear(sink, h, w_down)
-            assert ran == (["mid"] if sliced_ours else ["vendor"]), (packed, M, ran)
+            # (a small matrix at up to 32 rows goes to the few-row kernel instead of the vendor's)
+            assert ran == (["mid"] if sliced_ours else ([] if M <= 32 else ["vendor"])), (packed, M, ran)
             assert torch.allclose((residual - r0).double(), h.double() @ w_down.double().T, atol=5e-2, rtol=3e-2)
 
 

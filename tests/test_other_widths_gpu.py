@@ -134,15 +134,18 @@ def test_partial_packing_takes_the_matrices_whose_rows_collide_and_changes_no_bi
     small shapes first, within a budget.  One layer at the 70B widths with room for 320 MB: the
     head (384 x 8192), o_proj (8192 x 8192) and qkv_proj (10240 x 8192) are packed, gate_up
     (57344 x 8192) does not fit, down_proj (8192 x 28672, rows 56 KB apart) does not qualify.
-    The logits are the bits of the model without any packed copy, and of the one with all."""
+    The logits are the bits of the model without any packed copy, and of the one with all:
+    a prompt of 40 rows and single tokens, which take the same kernels with and without a packed
+    copy (at 17 to 32 rows and beyond 64 a matrix without one goes to the vendor's product,
+    whose sums round differently)."""
     from kvcore_amd.engine.runner import build_model
     from kvcore_amd.weights.loader import write_random_model
 
     cfg = SHAPES["70b"]
     folder = write_random_model(tmp_path / "w70", cfg, seed=5, device="cuda:0")
-    tokens = random_tokens(40, cfg["vocab_size"], seed=9)
-    steps = [{"step": 0, "entries": [{"id": "r", "tokens": tokens[:30], "want": [29]}], "end": []}]
-    steps += [{"step": i + 1, "entries": [{"id": "r", "tokens": [tokens[30 + i]], "want": [0]}], "end": []}
+    tokens = random_tokens(50, cfg["vocab_size"], seed=9)
+    steps = [{"step": 0, "entries": [{"id": "r", "tokens": tokens[:40], "want": [39]}], "end": []}]
+    steps += [{"step": i + 1, "entries": [{"id": "r", "tokens": [tokens[40 + i]], "want": [0]}], "end": []}
               for i in range(10)]
     rows = {}
     for mode in ("none", "partial", "all"):
