@@ -83,6 +83,9 @@ def parse_args():
     p.add_argument("--pack-weights", action=argparse.BooleanOptionalAction, default=None,
                    help="second copy of the weights in the order decode steps stream them "
                         "(default: where the device has room, as the engine decides)")
+    p.add_argument("--sampling", default=None, metavar="T[,K[,P]]",
+                   help="sample with this temperature, top-k and top-p (seeded) instead of greedily; "
+                        "not the contract's line: say so with --no-points")
     p.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     p.add_argument("--only-prefill", action="store_true",
                    help="run only the 2,048-token prefill (for profiling); prints its own line")
@@ -300,11 +303,23 @@ def main() -> int:
             check.update(check_prefill(cfg, dtype, args.dtype, args.page_size))
         print(f"[bench] check: {check}", file=sys.stderr, flush=True)
 
+    sampling = {"temperature": 0.0}
+    if args.sampling:
+        if not args.no_points:
+            print("bench.py: --sampling is not the contract's greedy line; pass --no-points with it", file=sys.stderr)
+            return 2
+        parts = [float(v) for v in args.sampling.split(",")]
+        sampling = {"temperature": parts[0], "seed": 1}
+        if len(parts) > 1:
+            sampling["top_k"] = int(parts[1])
+        if len(parts) > 2:
+            sampling["top_p"] = parts[2]
+
     def new_request(n_prompt, n_new, eng=None):
         counter[0] += 1
         rid = f"bench-{counter[0]}"
         ids = [rng.randrange(vocab) for _ in range(n_prompt)]
-        (eng or engine).add_request(rid, SamplingParams(max_tokens=n_new, temperature=0.0, ignore_eos=True),
+        (eng or engine).add_request(rid, SamplingParams(max_tokens=n_new, ignore_eos=True, **sampling),
                                     prompt_token_ids=ids)
         return rid
 
