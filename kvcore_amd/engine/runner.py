@@ -467,7 +467,7 @@ class ModelRunner:
         def run(keep: list | None = None) -> torch.Tensor:
             ctx = self._context(bucket, bucket, [1] * bucket, [plan_len] * bucket, 1, plan_len)
             hidden = self.model.forward(ctx)
-            logits = self.model.compute_logits(ctx, hidden, self._dev["logit_rows"], bucket)
+            logits = self.model.compute_logits(ctx, hidden, self._dev["logit_rows"], bucket, every_row=True)
             if keep is not None:  # nothing made in here dies before the capture has ended
                 keep.extend((ctx, hidden, logits))
             return logits

@@ -261,14 +261,18 @@ class DecoderModel:
         return hidden
 
     def compute_logits(self, ctx: StepContext, hidden: torch.Tensor, rows: torch.Tensor,
-                       num_rows: int) -> torch.Tensor:
-        """float32 ``[S, V]`` at the flattened token indices ``rows[:S]``."""
+                       num_rows: int, every_row: bool = False) -> torch.Tensor:
+        """float32 ``[S, V]`` at the flattened token indices ``rows[:S]``; ``every_row`` says
+        that these are simply all ``S`` rows of ``hidden`` in order, which saves the copy."""
         H, V = self.spec.hidden_size, self.spec.vocab_size
         # a row per request that samples, as a rule: room for all of them at once, so that a
         # batch that fills up step by step does not make these grow (and drop the graphs)
         room = ctx.buffers.seq_capacity
-        picked = ctx.buffers.get("head_rows", num_rows, H, self.dtype, reserve=room)
-        ops.gather_rows(picked, hidden, rows[:num_rows])
+        if every_row and hidden.shape == (num_rows, H) and hidden.dtype == self.dtype and hidden.is_contiguous():
+            picked = hidden
+        else:
+            picked = ctx.buffers.get("head_rows", num_rows, H, self.dtype, reserve=room)
+            ops.gather_rows(picked, hidden, rows[:num_rows])
         logits = ctx.buffers.get("logits", num_rows, V, torch.float32, reserve=room)
         self.head.forward(logits, picked, ctx)
         return logits
