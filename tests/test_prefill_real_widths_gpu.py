@@ -190,3 +190,56 @@ def test_the_end_of_the_prompt_in_small_portions_beside_decoding_requests(wide, 
     compare_rounding_noise(got, expects, what=WHAT)
     assert session.manager.live_requests() == []
     assert all(v.startswith("prefill_attention_kernel<128,") for v in spy.prefill) and spy.prefill
+
+
+def test_decode_steps_of_a_hundred_and_more_requests(wide, monkeypatch):
+    """Steps of single tokens for 190, 150, 120 and 90 requests at the 8B widths: the kernels
+    that share their rows through LDS with twelve, eight and six tiles of rows a wave (the
+    products cut along K up to 192 rows, the gated one up to 128), the vendor's product for the
+    rest.  Every decoded position of every request against the plain implementation."""
+    from kvcore_amd.ops import library as ops
+
+    folder, cfg, weights, model, _, _ = wide
+    live_after = [190, 150, 120, 90]
+    seqs = {}
+    for i in range(live_after[0]):
+        alive = sum(1 for n in live_after if i < n)
+        seqs[f"q{i}"] = random_tokens(2 + i % 4 + alive, cfg["vocab_size"], seed=900 + i)
+    expect = {rid: plain.llama_forward(cfg, weights, toks, dtype=torch.float32).double() for rid, toks in seqs.items()}
+    mid_rows, gated_rows = [], []
+    real_mid = ops.gemm_mid
+
+    def spy_mid(out, x, *a, **kw):
+        (gated_rows if kw.get("mode") == 1 else mid_rows).append(x.shape[0])
+        return real_mid(out, x, *a, **kw)
+
+    monkeypatch.setattr(ops, "gemm_mid", spy_mid)
+    vendor_rows = []
+    real_mm = torch.mm
+    monkeypatch.setattr(torch, "mm", lambda x, w, **kw: (vendor_rows.append(x.shape[0]), real_mm(x, w, **kw))[1])
+    total = sum(-(-len(t) // 64) * 64 for t in seqs.values())
+    session = session_for(folder, torch.bfloat16, PAGE, max_tokens=total, max_num_seqs=192, model=model)
+    ids = list(seqs)
+    fed = {r: len(seqs[r]) - sum(1 for n in live_after if int(r[1:]) < n) for r in ids}
+    steps, k = [], 0
+    for lo in range(0, len(ids), 10):  # prompts, ten requests a step
+        steps.append({"step": k, "end": [], "entries": [
+            {"id": r, "tokens": seqs[r][:fed[r]], "want": [fed[r] - 1]} for r in ids[lo:lo + 10]]})
+        k += 1
+    for j, n in enumerate(live_after):
+        live = ids[:n]
+        nxt = live_after[j + 1] if j + 1 < len(live_after) else 0
+        steps.append({"step": k, "end": live[nxt:], "entries": [
+            {"id": r, "tokens": [seqs[r][fed[r]]], "want": [0]} for r in live]})
+        k += 1
+        for r in live:
+            fed[r] += 1
+    got = collect(session, steps)
+    assert all(fed[r] == len(seqs[r]) for r in ids)
+    assert len(got) == len(ids) + sum(live_after)
+    compare_rounding_noise(got, expect, what="decode steps of 90 to 190 rows at 8B widths")
+    # padded to the sizes at which such steps are captured: 192, 160, 128 and 96 rows
+    assert {192, 160, 128, 96} <= set(mid_rows), sorted(set(mid_rows))
+    assert {128, 96} <= set(gated_rows) and not {192, 160} & set(gated_rows), sorted(set(gated_rows))
+    assert {192, 160} <= set(vendor_rows), sorted(set(vendor_rows))
+    assert session.manager.live_requests() == []
